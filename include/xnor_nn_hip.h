@@ -1,0 +1,79 @@
+/*
+ * Extensions of the MI355X / gfx950 build of xnor_nn.  None of these exist in
+ * mistler/xnor_nn; each comment names the reference behaviour it stands in for.
+ *
+ * Why they exist: in the reference, slots 3..8 of xnor_nn_resources_t are host memory
+ * that callers and tests read directly (reference test/gtest/test_binarization.cpp:72-77).
+ * Here they are device memory in a GPU-friendly word layout, so reading them goes
+ * through the export helpers below, which return the reference's canonical host layout.
+ */
+#ifndef XNOR_NN_HIP_H
+#define XNOR_NN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "xnor_nn_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* HIP stream (a hipStream_t passed as void*) on which the executors of this descriptor
+ * launch; default: the null stream.  With device pointers in slots 0..2 the executors
+ * only enqueue work and return; with host pointers they copy synchronously.
+ * Stands in for the reference's implicit "runs on the calling thread + OpenMP team". */
+xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *stream);
+
+/* Block until everything enqueued by this descriptor's executors has finished. */
+xnor_nn_status_t xnor_nn_hip_synchronize(const xnor_nn_convolution_t *c);
+
+/* Bytes per packed word of the reference's CPU layout for this shape: 2 while
+ * ic*kh*kw < 32767, else 4 (reference src/implementation.cpp:17-22,
+ * src/convolution_traits.hpp:29-56).  Only the export helpers depend on it. */
+int xnor_nn_hip_canonical_bici(const xnor_nn_convolution_t *c);
+
+/* Copy res[bin_src] to host memory in the reference's layout
+ * (reference src/bcast_binarize_data.cpp:43-73):
+ *   dst[((mb*IH+ih)*IW+iw)*ABIC + b], bit (7-j) = 1 iff channel 8b+j has its sign bit
+ *   clear; channels >= IC and pad bytes are 0; ABIC = ceil(ceil(IC/8)/bici)*bici.
+ * dst_bytes must be MB*IH*IW*ABIC. */
+xnor_nn_status_t xnor_nn_hip_export_bin_src(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, void *dst, size_t dst_bytes);
+
+/* Copy res[bin_weights] to host memory in the reference's layout for a CPU that packs
+ * `oci` filters per block (reference src/bcast_binarize_weights.cpp:54-93; oci = 16 for
+ * int16 words / 8 for int32 words on a 256-bit CPU):
+ *   dst[((((oco*KH+kh)*KW+kw)*ICO+ico)*oci+i)*bici + b], MSB-first, channels >= IC are 1.
+ * oc must be a multiple of oci.  dst_bytes must be (OC/oci)*KH*KW*ICO*oci*bici. */
+xnor_nn_status_t xnor_nn_hip_export_bin_weights(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int oci, void *dst, size_t dst_bytes);
+
+/* Copy one of the float resources (xnor_nn_resource_alpha, _a, _k) to host memory,
+ * shaped as in the reference (alpha[OC], a[MB][IH][IW], k[MB][OH][OW]). */
+xnor_nn_status_t xnor_nn_hip_export_floats(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int slot, float *dst, size_t dst_bytes);
+
+/* Copy res[operations_count] to host memory as int32[OH][OW]
+ * (reference src/bcast_binarize_weights.cpp:126-142 stores int16 or int32). */
+xnor_nn_status_t xnor_nn_hip_export_operations_count(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int32_t *dst, size_t dst_bytes);
+
+/* Run the convolution stage but store the raw integer accumulators
+ * popc[mb][oc][oh][ow] (int32, host or device pointer) instead of the scaled floats:
+ * the `d_arr` values of reference src/default/bcast_convolution_default.cpp:64-91.
+ * Needs res[bin_src] and res[bin_weights]; same kernel as forward, other epilogue. */
+xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int32_t *popc);
+
+/* Name of the kernel variant an executor of this descriptor launches (stage: one of
+ * xnor_nn_operation_t), e.g. "conv_xnor_popc<XW=12,Q=16>"; the counterpart of the
+ * reference's XNOR_NN_VERBOSE line (reference src/utils/convolution_logger.hpp:99-152).
+ * Returns the length written (without terminator). */
+int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage,
+        char *buf, size_t buf_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XNOR_NN_HIP_H */

@@ -1,0 +1,213 @@
+"""Parity of the HIP path against the CPU oracle and the committed digests of the upstream
+library's outputs.  Everything goes through the C ABI of libxnor_nn.so.
+
+Bar: packed tensors, operation counts and integer popcount accumulators bit-exact; the
+float tensors (a, k, alpha, dst) are computed in the reference's summation order and are
+asserted bit-exact as well, which is stricter than the 1e-5 relative tolerance allowed for
+them (the tolerance check is kept in `check_floats` for the error message only)."""
+import numpy as np
+import pytest
+
+import shapes
+from util import oracle_shape, relative_error, sha256
+from xnor_nn_amd import Convolution, capi, synth
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-5
+
+NCHW = (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW)
+
+
+def make(d, w, fmts=NCHW):
+    return Convolution(capi.ALGORITHM_BCAST, fmts[0], fmts[1], fmts[2],
+                       d["mb"], d["oc"], d["ic"], d["ih"], d["iw"], d["kh"], d["kw"],
+                       d["sh"], d["sw"], d["ph"], d["pw"], w)
+
+
+def check_floats(name, got, want):
+    err = relative_error(got, want)
+    assert err <= REL_TOL, "%s: relative error %.3e > %.0e" % (name, err, REL_TOL)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), \
+        "%s within tolerance (%.3e) but not bit-identical" % (name, err)
+
+
+def run_and_compare(oracle, d, x, w, fmts=NCHW, device_tensors=False, gpu=None):
+    """Full pipeline on the GPU vs the oracle, every intermediate."""
+    s = oracle_shape(oracle, d, fmts)
+    want = oracle.forward(s, x, w)
+    dshape = want["dst"].shape
+    if device_tensors:
+        import torch
+        xt = torch.from_numpy(x).to(gpu)
+        wt = torch.from_numpy(w).to(gpu)
+        dt = torch.empty(dshape, dtype=torch.float32, device=gpu)
+        conv = make(d, wt, fmts)
+        conv.forward(xt, dt)
+        conv.synchronize()
+        dst = dt.cpu().numpy()
+    else:
+        dst = np.full(dshape, np.nan, dtype=np.float32)
+        conv = make(d, w, fmts)
+        conv.forward(x, dst)
+    assert np.array_equal(conv.export_bin_src(), want["bin_src"]), "bin_src"
+    assert np.array_equal(conv.export_operations_count(), want["opc"]), "operations_count"
+    if d["oc"] % oracle.default_oci(s) == 0:
+        assert np.array_equal(conv.export_bin_weights(), want["bin_weights"]), "bin_weights"
+    check_floats("alpha", conv.export_floats(capi.RES_ALPHA), want["alpha"])
+    check_floats("a", conv.export_floats(capi.RES_A), want["a"])
+    check_floats("k", conv.export_floats(capi.RES_K), want["k"])
+    assert np.array_equal(conv.forward_popcount(), want["popc"]), "popcount accumulators"
+    check_floats("dst", dst, want["dst"])
+    conv.close()
+    return dst, want
+
+
+@pytest.mark.parametrize("t", shapes.COMPARE_WITH_REFERENCE, ids=shapes.shape_id)
+def test_reference_test_matrix(oracle, golden, t):
+    """The shape matrix and closed-form inputs of the reference's differential test
+    (reference test/gtest/test_convolution_compare_with_reference.cpp:9-27,82-217), host
+    pointers like the reference's tests; also against the upstream digests."""
+    d = shapes.as_dims(t)
+    x = synth.reference_test_src(d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.reference_test_weights(d["oc"], d["ic"], d["kh"], d["kw"])
+    dst, _ = run_and_compare(oracle, d, x, w)
+    assert sha256(dst) == golden["reference_test_shapes"][shapes.shape_id(t)]["sha256"]["dst"]
+
+
+@pytest.mark.parametrize("name,mb", [
+    ("alexnet_conv4_mb1", None), ("alexnet_conv4_mb256", 16), ("alexnet_conv2_mb128", 4),
+    ("resnet_3x3_mb64", 2), ("vgg_512_mb32", 2)])
+def test_workloads_reduced_batch(oracle, gpu, name, mb):
+    """The five benchmark workloads at a small batch, device-resident tensors."""
+    d, x, w = synth.make_workload(name, mb)
+    run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+
+
+@pytest.mark.parametrize("name", list(synth.WORKLOADS))
+def test_workloads_full_size_digests(oracle, golden, gpu, name):
+    """Benchmark sizes: every tensor the GPU produced hashes to what the upstream library
+    produced on the same seeded inputs (tests/golden/golden.json), and to the oracle."""
+    import torch
+    d, x, w = synth.make_workload(name)
+    g = golden["workloads"][name]["sha256"]
+    xt = torch.from_numpy(x).to(gpu)
+    wt = torch.from_numpy(w).to(gpu)
+    dt = torch.empty((d["mb"], d["oc"], d["ih"], d["iw"]), dtype=torch.float32, device=gpu)
+    conv = make(d, wt)
+    conv.forward(xt, dt)
+    conv.synchronize()
+    assert sha256(conv.export_bin_src()) == g["bin_src"]
+    assert sha256(conv.export_bin_weights()) == g["bin_weights"]
+    assert sha256(conv.export_operations_count()) == g["opc"]
+    assert sha256(conv.export_floats(capi.RES_ALPHA)) == g["alpha"]
+    assert sha256(conv.export_floats(capi.RES_A)) == g["a"]
+    assert sha256(conv.export_floats(capi.RES_K)) == g["k"]
+    dst = dt.cpu().numpy()
+    assert sha256(dst) == g["dst"]
+    # integer accumulators against the oracle, and the size-independent identity
+    # 2*popc - n == dst / (alpha*k) up to the two roundings
+    s = oracle_shape(oracle, d)
+    want = oracle.forward(s, x, w)
+    pt = torch.empty((d["mb"], d["oc"], d["ih"], d["iw"]), dtype=torch.int32, device=gpu)
+    conv.forward_popcount(pt)
+    conv.synchronize()
+    assert np.array_equal(pt.cpu().numpy(), want["popc"])
+    assert np.array_equal(dst.view(np.uint32), want["dst"].view(np.uint32))
+    conv.close()
+
+
+@pytest.mark.parametrize("fmts", [
+    (capi.FMT_NHWC, capi.FMT_OIHW, capi.FMT_NCHW),
+    (capi.FMT_NCHW, capi.FMT_HWIO, capi.FMT_NCHW),
+    (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC),
+    (capi.FMT_NHWC, capi.FMT_HWIO, capi.FMT_NHWC),
+])
+@pytest.mark.parametrize("t", [(3, 40, 32, 9, 11, 3, 3, 1, 1, 1, 1),
+                               (2, 96, 48, 13, 13, 5, 5, 1, 1, 2, 2)], ids=shapes.shape_id)
+def test_tensor_formats(oracle, fmts, t):
+    """NHWC input, HWIO weights and NHWC output (reference
+    src/bcast_binarize_data.cpp:56-57, src/bcast_binarize_weights.cpp:71-72,
+    src/default/bcast_convolution_default.cpp:97-99)."""
+    d = shapes.as_dims(t)
+    x = synth.normal(31, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(32, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    if fmts[0] == capi.FMT_NHWC:
+        x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    if fmts[1] == capi.FMT_HWIO:
+        w = np.ascontiguousarray(w.transpose(2, 3, 1, 0))
+    run_and_compare(oracle, d, x, w, fmts)
+
+
+@pytest.mark.parametrize("t", [
+    (1, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0),        # smallest possible problem
+    (2, 5, 3, 4, 6, 3, 3, 1, 1, 1, 1),        # oc below one filter group
+    (1, 70, 20, 7, 5, 3, 3, 2, 2, 1, 1),      # stride 2, ic and oc ragged
+    (3, 33, 17, 6, 6, 5, 5, 1, 1, 2, 2),      # one bit past a word
+    (1, 1100, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # more than 1024 channels
+    (1, 3700, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # ic*kh*kw > 32767: int32 words upstream
+    (5, 64, 64, 5, 9, 1, 1, 1, 1, 0, 0),      # 1x1 filter
+    (2, 16, 32, 8, 8, 3, 3, 1, 1, 0, 0),      # no padding
+    (1, 24, 16, 12, 12, 7, 7, 3, 3, 3, 3),    # big filter, stride 3
+], ids=shapes.shape_id)
+def test_edge_shapes(oracle, t):
+    d = shapes.as_dims(t)
+    x = synth.normal(41, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::5] = 0.0
+    x.ravel()[2::9] = -0.0
+    w = synth.normal(42, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    w.ravel()[::13] = -0.0
+    run_and_compare(oracle, d, x, w)
+
+
+def test_known_answer_forward_on_gpu():
+    """The reference's 18 precomputed outputs
+    (reference test/gtest/test_convolution_reference_forward.cpp:20-73), tolerance 1e-3."""
+    from test_oracle import KA_DIMS, KA_DST, KA_SRC, KA_W
+    conv = make(KA_DIMS, KA_W)
+    dst = np.zeros((1, 2, 3, 3), np.float32)
+    conv.forward(KA_SRC, dst)
+    assert np.allclose(dst, KA_DST, atol=1e-3, rtol=0)
+    conv.close()
+
+
+def test_calculate_k_alone_matches_fused_path(oracle, gpu):
+    """calculate_k called without a preceding binarize_data reads the input itself; both
+    routes give the same bits."""
+    import torch
+    d, x, w = synth.make_workload("alexnet_conv4_mb256", 8)
+    s = oracle_shape(oracle, d)
+    a_want, k_want = oracle.calculate_k(s, x)
+    xt = torch.from_numpy(x).to(gpu)
+    conv = make(d, w)
+    conv.stage("calculate_k", src=xt)
+    assert np.array_equal(conv.export_floats(capi.RES_A), a_want)
+    assert np.array_equal(conv.export_floats(capi.RES_K), k_want)
+    conv.stage("binarize_data", src=xt)
+    conv.stage("calculate_k", src=xt)
+    assert np.array_equal(conv.export_floats(capi.RES_K), k_want)
+    conv.close()
+
+
+def test_linearity_of_scaling_at_full_size(gpu):
+    """Size-independent property at benchmark size: scaling the input by 2 leaves the
+    packed bits and popcounts unchanged and doubles dst exactly (k is linear in |x| and
+    powers of two commute with rounding)."""
+    import torch
+    d, x, w = synth.make_workload("alexnet_conv4_mb256")
+    xt = torch.from_numpy(x).to(gpu)
+    wt = torch.from_numpy(w).to(gpu)
+    shape = (d["mb"], d["oc"], d["ih"], d["iw"])
+    y1 = torch.empty(shape, dtype=torch.float32, device=gpu)
+    y2 = torch.empty(shape, dtype=torch.float32, device=gpu)
+    conv = make(d, wt)
+    conv.forward(xt, y1)
+    b1 = conv.export_bin_src()
+    conv.forward(xt * 2, y2)
+    conv.synchronize()
+    assert np.array_equal(conv.export_bin_src(), b1)
+    assert torch.equal(y2, y1 * 2)
+    conv.close()

@@ -99,6 +99,14 @@ def load():
             raise RuntimeError(
                 "%s is missing: build it with `python -m xnor_nn_amd.build` "
                 "(hipcc --offload-arch=gfx950); there is no CPU fallback" % path)
+        # A process must hold ONE HIP runtime.  PyTorch ships its own copy (same soname as
+        # the system one): when torch is imported first, the dynamic loader resolves this
+        # library's dependency to that copy; the other order would load a second runtime
+        # and leave torch without a device.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = C.CDLL(path)
         bind(lib, CORE_SYMBOLS)
         bind(lib, HIP_SYMBOLS)

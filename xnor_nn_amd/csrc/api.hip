@@ -1,0 +1,450 @@
+// C entry points of libxnor_nn.so (include/xnor_nn.h, include/xnor_nn_hip.h): descriptor
+// setup, device resources, the four stage executors and the export helpers.
+//
+// Host side only; every kernel lives in the kernels_*.hip files behind the launch_*
+// functions of plan.hpp.  There is no CPU implementation of any stage: when no GPU is
+// usable the executors report xnor_nn_error_memory.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "plan.hpp"
+#include "xnor_nn_hip.h"
+
+using namespace xnor_hip;
+
+namespace {
+
+bool is_data_format(int f) {
+    return f == xnor_nn_data_format_nchw || f == xnor_nn_data_format_nhwc;
+}
+bool is_weights_format(int f) {
+    return f == xnor_nn_weights_format_oihw || f == xnor_nn_weights_format_hwio;
+}
+
+size_t src_elems(const Geometry &g) { return (size_t)g.mb * g.ic * g.ih * g.iw; }
+size_t weights_elems(const Geometry &g) { return (size_t)g.oc * g.ic * g.kh * g.kw; }
+size_t dst_elems(const Geometry &g) { return (size_t)g.mb * g.oc * g.oh * g.ow; }
+
+// True when a kernel can dereference p (device or managed allocation).
+bool on_device(const void *p) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError(); // plain host memory: clear the sticky error
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+// Device view of a user tensor the kernels read: the pointer itself, or a staged copy.
+xnor_nn_status_t stage_in(State *st, void **slot, const void *user, size_t bytes,
+        const void **dev) {
+    if (on_device(user)) { *dev = user; return xnor_nn_success; }
+    if (!*slot && hipMalloc(slot, bytes) != hipSuccess) return xnor_nn_error_memory;
+    if (hipMemcpyAsync(*slot, user, bytes, hipMemcpyHostToDevice, st->stream) != hipSuccess)
+        return xnor_nn_error_memory;
+    // the host buffer may be pageable: the copy must have left it before we return
+    if (hipStreamSynchronize(st->stream) != hipSuccess) return xnor_nn_error_memory;
+    *dev = *slot;
+    return xnor_nn_success;
+}
+
+xnor_nn_status_t unimplemented_stage(const xnor_nn_convolution_t *, xnor_nn_resources_t) {
+    return xnor_nn_unimplemented;
+}
+
+// ---- stage 1 --------------------------------------------------------------------------
+// Replaces reference src/bcast_binarize_data.cpp:13-76 (same null checks, same
+// "unimplemented" for an unknown format).
+xnor_nn_status_t exec_binarize_data(const xnor_nn_convolution_t *c, xnor_nn_resources_t res) {
+    if (c == nullptr || res[xnor_nn_resource_user_src] == nullptr
+            || res[xnor_nn_resource_bin_src] == nullptr)
+        return xnor_nn_error_invalid_input;
+    if (!is_data_format(c->src_format)) return xnor_nn_unimplemented;
+    State *st = state_of(c);
+    const void *x = nullptr;
+    xnor_nn_status_t rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
+            src_elems(st->g) * sizeof(float), &x);
+    if (rc != xnor_nn_success) return rc;
+    float *a = static_cast<float *>(res[xnor_nn_resource_a]); // optional by-product
+    if (st->verbose) printf("xnor_nn exec binarize_data: %s\n", binarize_kernel_name(st->g));
+    if (launch_binarize_data(st->g, static_cast<const float *>(x),
+                static_cast<uint32_t *>(res[xnor_nn_resource_bin_src]), a, st->stream)
+            != hipSuccess)
+        return xnor_nn_error_memory;
+    st->a_ready_src = a ? res[xnor_nn_resource_user_src] : nullptr;
+    st->a_ready_buf = a;
+    return xnor_nn_success;
+}
+
+// ---- stage 2 --------------------------------------------------------------------------
+// Replaces reference src/bcast_calculate_k.cpp:13-88.  When the preceding
+// binarize_data call on the same src/a buffers already produced mean|x|, only the box
+// filter runs; otherwise the input is read here.
+xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resources_t res) {
+    if (c == nullptr || res[xnor_nn_resource_user_src] == nullptr
+            || res[xnor_nn_resource_a] == nullptr || res[xnor_nn_resource_k] == nullptr)
+        return xnor_nn_error_invalid_input;
+    if (!is_data_format(c->src_format)) return xnor_nn_unimplemented;
+    State *st = state_of(c);
+    float *a = static_cast<float *>(res[xnor_nn_resource_a]);
+    const bool a_ready = st->a_ready_src == res[xnor_nn_resource_user_src]
+        && st->a_ready_buf == a && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr;
+    st->a_ready_src = st->a_ready_buf = nullptr; // one-shot
+    if (!a_ready) {
+        const void *x = nullptr;
+        xnor_nn_status_t rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
+                src_elems(st->g) * sizeof(float), &x);
+        if (rc != xnor_nn_success) return rc;
+        if (launch_mean_abs(st->g, static_cast<const float *>(x), a, st->stream) != hipSuccess)
+            return xnor_nn_error_memory;
+    }
+    if (st->verbose)
+        printf("xnor_nn exec calculate_k: %sbox_filter_kernel\n", a_ready ? "" : "mean_abs + ");
+    if (launch_box_filter(st->g, a, static_cast<float *>(res[xnor_nn_resource_k]), st->stream)
+            != hipSuccess)
+        return xnor_nn_error_memory;
+    return xnor_nn_success;
+}
+
+// ---- weights --------------------------------------------------------------------------
+// Replaces reference src/bcast_binarize_weights.cpp:13-145.
+xnor_nn_status_t exec_binarize_weights(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res) {
+    if (c == nullptr || res[xnor_nn_resource_user_weights] == nullptr
+            || res[xnor_nn_resource_bin_weights] == nullptr
+            || res[xnor_nn_resource_operations_count] == nullptr
+            || res[xnor_nn_resource_alpha] == nullptr)
+        return xnor_nn_error_invalid_input;
+    if (!is_weights_format(c->weights_format)) return xnor_nn_unimplemented;
+    State *st = state_of(c);
+    const void *w = nullptr;
+    xnor_nn_status_t rc = stage_in(st, &st->stage_weights, res[xnor_nn_resource_user_weights],
+            weights_elems(st->g) * sizeof(float), &w);
+    if (rc != xnor_nn_success) return rc;
+    if (st->verbose) printf("xnor_nn exec binarize_weights: pack/alpha/op_count kernels\n");
+    if (launch_binarize_weights(st->g, static_cast<const float *>(w),
+                static_cast<uint32_t *>(res[xnor_nn_resource_bin_weights]),
+                static_cast<float *>(res[xnor_nn_resource_alpha]),
+                static_cast<int32_t *>(res[xnor_nn_resource_operations_count]), st->stream)
+            != hipSuccess)
+        return xnor_nn_error_memory;
+    return xnor_nn_success;
+}
+
+// ---- stage 3 --------------------------------------------------------------------------
+xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resources_t res,
+        void *user_out, bool raw) {
+    State *st = state_of(c);
+    const size_t bytes = dst_elems(st->g) * 4;
+    void *out = user_out;
+    const bool direct = on_device(user_out);
+    if (!direct) {
+        if (!st->stage_dst && hipMalloc(&st->stage_dst, bytes) != hipSuccess)
+            return xnor_nn_error_memory;
+        out = st->stage_dst;
+    }
+    if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
+    if (launch_convolution(st->g, static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]),
+                static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]),
+                static_cast<const float *>(res[xnor_nn_resource_alpha]),
+                static_cast<const float *>(res[xnor_nn_resource_k]),
+                static_cast<const int32_t *>(res[xnor_nn_resource_operations_count]),
+                raw ? nullptr : static_cast<float *>(out),
+                raw ? static_cast<int32_t *>(out) : nullptr, st->stream) != hipSuccess)
+        return xnor_nn_error_memory;
+    if (!direct) {
+        if (hipMemcpyAsync(user_out, out, bytes, hipMemcpyDeviceToHost, st->stream) != hipSuccess
+                || hipStreamSynchronize(st->stream) != hipSuccess)
+            return xnor_nn_error_memory;
+    }
+    return xnor_nn_success;
+}
+
+// Replaces reference src/default/bcast_convolution_default.cpp:14-108 / :110-216 and the
+// ISA-specific kernels selected in reference src/bcast_convolution.cpp:93-116.
+xnor_nn_status_t exec_forward(const xnor_nn_convolution_t *c, xnor_nn_resources_t res) {
+    if (c == nullptr || res[xnor_nn_resource_bin_src] == nullptr
+            || res[xnor_nn_resource_bin_weights] == nullptr
+            || res[xnor_nn_resource_user_dst] == nullptr
+            || res[xnor_nn_resource_k] == nullptr
+            || res[xnor_nn_resource_alpha] == nullptr
+            || res[xnor_nn_resource_operations_count] == nullptr)
+        return xnor_nn_error_invalid_input;
+    if (!is_data_format(c->dst_format)) return xnor_nn_unimplemented;
+    return run_convolution(c, res, res[xnor_nn_resource_user_dst], false);
+}
+
+xnor_nn_status_t to_host(const xnor_nn_convolution_t *c, const void *dev, void *dst,
+        size_t bytes) {
+    State *st = state_of(c);
+    if (hipMemcpyAsync(dst, dev, bytes, hipMemcpyDeviceToHost, st->stream) != hipSuccess
+            || hipStreamSynchronize(st->stream) != hipSuccess)
+        return xnor_nn_error_memory;
+    return xnor_nn_success;
+}
+
+int canonical_bici(const Geometry &g) { return (g.ic * g.kh * g.kw < 32767) ? 2 : 4; }
+int div_up(int a, int b) { return (a + b - 1) / b; }
+
+bool bcast_descriptor(const xnor_nn_convolution_t *c) {
+    return c != nullptr && c->state != nullptr && c->algorithm == xnor_nn_algorithm_bcast;
+}
+
+} // namespace
+
+extern "C" {
+
+void xnor_nn_get_status_message(char *msg, xnor_nn_status_t status) {
+    const char *text = "unimplemented";
+    switch (status) {
+    case xnor_nn_success: text = "success"; break;
+    case xnor_nn_error_memory: text = "memory_error"; break;
+    case xnor_nn_error_invalid_input: text = "bad_input"; break;
+    case xnor_nn_unimplemented: text = "unimplemented"; break;
+    }
+    strcpy(msg, text);
+}
+
+xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
+        const xnor_nn_algorithm_t algorithm,
+        const xnor_nn_tensor_format_t src_fmt,
+        const xnor_nn_tensor_format_t weights_fmt,
+        const xnor_nn_tensor_format_t dst_fmt,
+        int mb, int oc, int ic, int ih, int iw,
+        int kh, int kw, int sh, int sw, int ph, int pw) {
+    c->algorithm = algorithm;
+    c->mb = mb;
+    c->ic = ic; c->ih = ih; c->iw = iw;
+    c->oc = oc;
+    // The reference derives BOTH extents from pw (src/common_convolution.cpp:16-17).
+    c->oh = (ih + 2 * pw - kh) / sh + 1;
+    c->ow = (iw + 2 * pw - kw) / sw + 1;
+    c->sh = sh; c->sw = sw;
+    c->kh = kh; c->kw = kw;
+    c->ph = ph; c->pw = pw;
+    c->src_format = src_fmt;
+    c->weights_format = weights_fmt;
+    c->dst_format = dst_fmt;
+    for (int i = xnor_nn_resource_internal; i < xnor_nn_resource_number; i++)
+        c->resource_size[i] = 0;
+    c->binarize_weights = unimplemented_stage;
+    c->binarize_data = unimplemented_stage;
+    c->calculate_k = unimplemented_stage;
+    c->forward = unimplemented_stage;
+    c->state = nullptr;
+
+    if (algorithm != xnor_nn_algorithm_bcast) return xnor_nn_success;
+
+    State *st = new (std::nothrow) State();
+    if (!st) return xnor_nn_success; // executors stay "unimplemented", like a failed match
+    Geometry &g = st->g;
+    g.mb = mb; g.ic = ic; g.ih = ih; g.iw = iw; g.oc = oc; g.oh = c->oh; g.ow = c->ow;
+    g.kh = kh; g.kw = kw; g.sh = sh; g.sw = sw; g.ph = ph; g.pw = pw;
+    g.src_fmt = src_fmt; g.w_fmt = weights_fmt; g.dst_fmt = dst_fmt;
+    g.xw = div_up(ic, 32);
+    g.q = pick_q(oc, g.xw);
+    g.ocb = div_up(oc, g.q);
+    g.ihw = ih * iw;
+    g.ohw = g.oh * g.ow;
+    g.npix_in = (uint32_t)mb * g.ihw;
+    g.npix_out = (uint32_t)mb * g.ohw;
+    g.div_ihw = FastDiv::make(g.ihw);
+    g.div_iw = FastDiv::make(iw);
+    g.div_ohw = FastDiv::make(g.ohw);
+    g.div_ow = FastDiv::make(g.ow);
+    const char *v = getenv("XNOR_NN_VERBOSE");
+    st->verbose = v && v[0] == '1';
+
+    // Byte sizes of the device buffers (the reference's are host sizes of its CPU layout,
+    // src/bcast_convolution.cpp:72-82).
+    c->resource_size[xnor_nn_resource_bin_src] = (size_t)g.npix_in * g.xw * 4;
+    c->resource_size[xnor_nn_resource_bin_weights] = (size_t)g.ocb * kh * kw * g.xw * g.q * 4;
+    c->resource_size[xnor_nn_resource_a] = (size_t)g.npix_in * 4;
+    c->resource_size[xnor_nn_resource_k] = (size_t)g.npix_out * 4;
+    c->resource_size[xnor_nn_resource_alpha] = (size_t)oc * 4;
+    c->resource_size[xnor_nn_resource_operations_count] = (size_t)g.ohw * 4;
+
+    c->binarize_weights = exec_binarize_weights;
+    c->binarize_data = exec_binarize_data;
+    c->calculate_k = exec_calculate_k;
+    c->forward = exec_forward;
+    c->state = st;
+    if (st->verbose)
+        printf("xnor_nn init: bcast gfx950 mb=%d ic=%d %dx%d oc=%d %dx%d k=%dx%d s=%dx%d "
+               "p=%dx%d words/pixel=%d conv=%s\n", mb, ic, ih, iw, oc, c->oh, c->ow, kh, kw,
+               sh, sw, ph, pw, g.xw, convolution_kernel_name(g));
+    return xnor_nn_success;
+}
+
+void xnor_nn_destroy_convolution(xnor_nn_convolution_t *c) {
+    if (c == nullptr || c->state == nullptr) return;
+    State *st = state_of(c);
+    if (st->stage_src) (void)hipFree(st->stage_src);
+    if (st->stage_weights) (void)hipFree(st->stage_weights);
+    if (st->stage_dst) (void)hipFree(st->stage_dst);
+    delete st;
+    c->state = nullptr;
+}
+
+xnor_nn_status_t xnor_nn_allocate_resources(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res) {
+    for (int i = xnor_nn_resource_internal; i < xnor_nn_resource_number; i++) {
+        void *p = nullptr;
+        // a zero-sized slot still gets a distinct non-null buffer, as aligned_alloc gives
+        const size_t bytes = c->resource_size[i] ? c->resource_size[i] : 4;
+        if (hipMalloc(&p, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            xnor_nn_free_resources(res);
+            return xnor_nn_error_memory;
+        }
+        res[i] = p;
+    }
+    return xnor_nn_success;
+}
+
+void xnor_nn_free_resources(xnor_nn_resources_t res) {
+    for (int i = xnor_nn_resource_internal; i < xnor_nn_resource_number; i++) {
+        if (res[i]) (void)hipFree(res[i]);
+        res[i] = nullptr;
+    }
+}
+
+void xnor_nn_binarize_weights_float(const xnor_nn_convolution_t *c,
+        const float *from, float *to) {
+    const size_t n = (size_t)c->oc * c->ic * c->kh * c->kw;
+    const size_t bytes = n * sizeof(float);
+    hipStream_t s = c->state ? state_of(c)->stream : nullptr;
+    const bool from_dev = on_device(from), to_dev = on_device(to);
+    float *dfrom = nullptr, *dto = nullptr, *scratch = nullptr;
+    bool ok = hipMalloc((void **)&scratch, 256 * sizeof(float)) == hipSuccess;
+    if (ok && !from_dev) ok = hipMalloc((void **)&dfrom, bytes) == hipSuccess
+        && hipMemcpy(dfrom, from, bytes, hipMemcpyHostToDevice) == hipSuccess;
+    if (ok && !to_dev) ok = hipMalloc((void **)&dto, bytes) == hipSuccess;
+    if (ok) ok = launch_weights_float(from_dev ? from : dfrom, to_dev ? to : dto, n, scratch, s)
+        == hipSuccess;
+    if (ok && !to_dev) ok = hipMemcpyAsync(to, dto, bytes, hipMemcpyDeviceToHost, s) == hipSuccess;
+    if (hipStreamSynchronize(s) != hipSuccess) ok = false;
+    if (!ok) fprintf(stderr, "xnor_nn_binarize_weights_float: HIP failure, output not written\n");
+    if (dfrom) (void)hipFree(dfrom);
+    if (dto) (void)hipFree(dto);
+    if (scratch) (void)hipFree(scratch);
+}
+
+// ---- include/xnor_nn_hip.h --------------------------------------------------------------
+
+xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *stream) {
+    if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
+    state_of(c)->stream = static_cast<hipStream_t>(stream);
+    return xnor_nn_success;
+}
+
+xnor_nn_status_t xnor_nn_hip_synchronize(const xnor_nn_convolution_t *c) {
+    if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
+    return hipStreamSynchronize(state_of(c)->stream) == hipSuccess ? xnor_nn_success
+                                                                   : xnor_nn_error_memory;
+}
+
+int xnor_nn_hip_canonical_bici(const xnor_nn_convolution_t *c) {
+    return (c->ic * c->kh * c->kw < 32767) ? 2 : 4;
+}
+
+xnor_nn_status_t xnor_nn_hip_export_bin_src(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, void *dst, size_t dst_bytes) {
+    if (!bcast_descriptor(c) || !res[xnor_nn_resource_bin_src] || !dst)
+        return xnor_nn_error_invalid_input;
+    const Geometry &g = state_of(c)->g;
+    const int bici = canonical_bici(g);
+    const int abic = div_up(div_up(g.ic, 8), bici) * bici;
+    if (dst_bytes != (size_t)g.npix_in * abic) return xnor_nn_error_invalid_input;
+    std::vector<uint32_t> words((size_t)g.npix_in * g.xw);
+    xnor_nn_status_t rc = to_host(c, res[xnor_nn_resource_bin_src], words.data(),
+            words.size() * 4);
+    if (rc != xnor_nn_success) return rc;
+    unsigned char *out = static_cast<unsigned char *>(dst);
+    for (size_t p = 0; p < g.npix_in; p++)
+        for (int b = 0; b < abic; b++) {
+            const int j = b / 4;
+            out[p * abic + b] = j < g.xw
+                ? (unsigned char)(words[p * g.xw + j] >> (24 - 8 * (b % 4))) : 0;
+        }
+    return xnor_nn_success;
+}
+
+xnor_nn_status_t xnor_nn_hip_export_bin_weights(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int oci, void *dst, size_t dst_bytes) {
+    if (!bcast_descriptor(c) || !res[xnor_nn_resource_bin_weights] || !dst || oci <= 0)
+        return xnor_nn_error_invalid_input;
+    const Geometry &g = state_of(c)->g;
+    if (g.oc % oci != 0) return xnor_nn_error_invalid_input;
+    const int bici = canonical_bici(g);
+    const int ico = div_up(div_up(g.ic, bici), 8);
+    const int taps = g.kh * g.kw;
+    const size_t need = (size_t)(g.oc / oci) * taps * ico * oci * bici;
+    if (dst_bytes != need) return xnor_nn_error_invalid_input;
+    std::vector<uint32_t> words((size_t)g.ocb * taps * g.xw * g.q);
+    xnor_nn_status_t rc = to_host(c, res[xnor_nn_resource_bin_weights], words.data(),
+            words.size() * 4);
+    if (rc != xnor_nn_success) return rc;
+    unsigned char *out = static_cast<unsigned char *>(dst);
+    for (int oc = 0; oc < g.oc; oc++)
+        for (int t = 0; t < taps; t++)
+            for (int b = 0; b < ico * bici; b++) {
+                const int j = b / 4;
+                unsigned char byte = 0xFF; // bytes past the device words: channels >= IC
+                if (j < g.xw) {
+                    const uint32_t w = words[(((size_t)(oc / g.q) * taps + t) * g.xw + j) * g.q
+                        + oc % g.q];
+                    byte = (unsigned char)(w >> (24 - 8 * (b % 4)));
+                }
+                const size_t at = ((((size_t)(oc / oci) * taps + t) * ico + b / bici) * oci
+                        + oc % oci) * bici + b % bici;
+                out[at] = byte;
+            }
+    return xnor_nn_success;
+}
+
+xnor_nn_status_t xnor_nn_hip_export_floats(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int slot, float *dst, size_t dst_bytes) {
+    if (!bcast_descriptor(c) || !dst) return xnor_nn_error_invalid_input;
+    if (slot != xnor_nn_resource_alpha && slot != xnor_nn_resource_a
+            && slot != xnor_nn_resource_k)
+        return xnor_nn_error_invalid_input;
+    if (!res[slot] || dst_bytes != c->resource_size[slot]) return xnor_nn_error_invalid_input;
+    return to_host(c, res[slot], dst, dst_bytes);
+}
+
+xnor_nn_status_t xnor_nn_hip_export_operations_count(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int32_t *dst, size_t dst_bytes) {
+    if (!bcast_descriptor(c) || !dst || !res[xnor_nn_resource_operations_count]
+            || dst_bytes != c->resource_size[xnor_nn_resource_operations_count])
+        return xnor_nn_error_invalid_input;
+    return to_host(c, res[xnor_nn_resource_operations_count], dst, dst_bytes);
+}
+
+xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
+        xnor_nn_resources_t res, int32_t *popc) {
+    if (!bcast_descriptor(c) || res[xnor_nn_resource_bin_src] == nullptr
+            || res[xnor_nn_resource_bin_weights] == nullptr || popc == nullptr)
+        return xnor_nn_error_invalid_input;
+    return run_convolution(c, res, popc, true);
+}
+
+int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage, char *buf,
+        size_t buf_bytes) {
+    if (!bcast_descriptor(c) || !buf || buf_bytes == 0) return 0;
+    const Geometry &g = state_of(c)->g;
+    const char *name = "";
+    switch (stage) {
+    case xnor_nn_operation_convolution_forward: name = convolution_kernel_name(g); break;
+    case xnor_nn_operation_binarize_data: name = binarize_kernel_name(g); break;
+    case xnor_nn_operation_calculate_k: name = "box_filter_kernel"; break;
+    case xnor_nn_operation_binarize_weights: name = "pack_weights_kernel"; break;
+    }
+    snprintf(buf, buf_bytes, "%s", name);
+    return (int)strlen(buf);
+}
+
+} // extern "C"

@@ -1,0 +1,128 @@
+// Once-per-weight-set stage: sign-bit packing of the filters, alpha = mean |w| per filter
+// and the per-output-pixel operation counts
+// (reference src/bcast_binarize_weights.cpp:54-142), plus the float sign(w)*mean(w)
+// helper (reference src/binarize_weights_float.cpp:3-25).  None of this is on the
+// per-forward path, so the kernels favour exact reference order over speed.
+#include "plan.hpp"
+
+namespace xnor_hip {
+
+namespace {
+
+__device__ __forceinline__ size_t w_index(const Geometry &g, int oc, int ic, int kh, int kw) {
+    if (g.w_fmt == xnor_nn_weights_format_oihw)
+        return (((size_t)oc * g.ic + ic) * g.kh + kh) * g.kw + kw;
+    return (((size_t)kh * g.kw + kw) * g.ic + ic) * g.oc + oc;
+}
+
+// One thread per packed word of the device layout [OCB][KH*KW][XW][Q].
+// Channels >= IC (and whole filters >= OC) are written as ones so that
+// popcount(xnor(0, 1)) adds nothing (reference src/bcast_binarize_weights.cpp:80-88).
+__global__ __launch_bounds__(256)
+void pack_weights_kernel(const float *__restrict__ w, uint32_t *__restrict__ bits,
+        const Geometry g) {
+    const int taps = g.kh * g.kw;
+    const size_t total = (size_t)g.ocb * taps * g.xw * g.q;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int qi = (int)(i % g.q);
+    const int j = (int)((i / g.q) % g.xw);
+    const int tap = (int)((i / ((size_t)g.q * g.xw)) % taps);
+    const int ob = (int)(i / ((size_t)g.q * g.xw * taps));
+    const int oc = ob * g.q + qi;
+    const int kh = tap / g.kw, kw = tap % g.kw;
+    uint32_t word = 0;
+    for (int b = 0; b < 32; b++) {
+        const int c = 32 * j + b;
+        uint32_t bit = 1u;
+        if (oc < g.oc && c < g.ic)
+            bit = (~__float_as_uint(w[w_index(g, oc, c, kh, kw)])) >> 31;
+        word = (word << 1) | bit;
+    }
+    bits[i] = word;
+}
+
+// alpha[oc] = sum over (ic, kh, kw), nested in that order, of fl(|w| * chw)
+// (reference src/bcast_binarize_weights.cpp:95-115).  One thread per filter.
+__global__ __launch_bounds__(64)
+void alpha_kernel(const float *__restrict__ w, float *__restrict__ alpha,
+        const Geometry g, const float chw) {
+    const int oc = blockIdx.x * blockDim.x + threadIdx.x;
+    if (oc >= g.oc) return;
+    float acc = 0.f;
+    for (int ic = 0; ic < g.ic; ic++)
+        for (int kh = 0; kh < g.kh; kh++)
+            for (int kw = 0; kw < g.kw; kw++)
+                acc = __fadd_rn(acc,
+                        __fmul_rn(__builtin_fabsf(w[w_index(g, oc, ic, kh, kw)]), chw));
+    alpha[oc] = acc;
+}
+
+// opc[oh][ow] = IC * number of in-bounds taps (reference
+// src/bcast_binarize_weights.cpp:126-142).
+__global__ __launch_bounds__(256)
+void op_count_kernel(int32_t *__restrict__ opc, const Geometry g) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= g.ohw) return;
+    const int oh = p / g.ow, ow = p % g.ow;
+    int taps = 0;
+    for (int kh = 0; kh < g.kh; kh++) {
+        const int ih = oh * g.sh - g.ph + kh;
+        if (ih < 0 || ih >= g.ih) continue;
+        for (int kw = 0; kw < g.kw; kw++) {
+            const int iw = ow * g.sw - g.pw + kw;
+            if (iw < 0 || iw >= g.iw) continue;
+            taps++;
+        }
+    }
+    opc[p] = taps * g.ic;
+}
+
+// Deterministic two-level sum for the float-weights helper: 256 partial sums, each over a
+// contiguous slice in index order, then a serial sum of the partials.
+constexpr int PARTS = 256;
+
+__global__ __launch_bounds__(PARTS)
+void partial_sum_kernel(const float *__restrict__ from, float *__restrict__ parts,
+        const size_t n) {
+    const size_t per = (n + PARTS - 1) / PARTS;
+    const size_t lo = threadIdx.x * per;
+    const size_t hi = lo + per < n ? lo + per : n;
+    float acc = 0.f;
+    for (size_t i = lo; i < hi; i++) acc += from[i];
+    parts[threadIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(256)
+void sign_times_mean_kernel(const float *__restrict__ from, float *__restrict__ to,
+        const float *__restrict__ parts, const size_t n, const float inv_n) {
+    float sum = 0.f;
+    for (int i = 0; i < PARTS; i++) sum += parts[i];
+    const float mean = sum * inv_n;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) to[i] = (from[i] >= 0.f ? 1.f : -1.f) * mean;
+}
+
+} // namespace
+
+hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *bits,
+        float *alpha, int32_t *opc, hipStream_t s) {
+    const size_t words = (size_t)g.ocb * g.kh * g.kw * g.xw * g.q;
+    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256),
+            0, s, w, bits, g);
+    const float chw = 1.f / (g.ic * g.kh * g.kw);
+    hipLaunchKernelGGL(alpha_kernel, dim3((g.oc + 63) / 64), dim3(64), 0, s, w, alpha, g, chw);
+    hipLaunchKernelGGL(op_count_kernel, dim3((g.ohw + 255) / 256), dim3(256), 0, s, opc, g);
+    return hipGetLastError();
+}
+
+// scratch: PARTS floats of device memory.
+hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
+        hipStream_t s) {
+    hipLaunchKernelGGL(partial_sum_kernel, dim3(1), dim3(PARTS), 0, s, from, scratch, n);
+    hipLaunchKernelGGL(sign_times_mean_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256),
+            0, s, from, to, scratch, n, 1.f / (float)n);
+    return hipGetLastError();
+}
+
+} // namespace xnor_hip

@@ -1,0 +1,90 @@
+// Launch plan and per-descriptor state of the gfx950 implementation.
+//
+// Takes the place of the reference's Implementation object behind c->state
+// (reference src/implementation.hpp:11-27, src/bcast_convolution.cpp:58-117): instead of
+// CPU blocking factors (BIC/ABIC/ICO/OCI/OCO) it records the device word layout, the
+// launch geometry, the stream and the staging buffers used when the caller hands over
+// host pointers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "xnor_nn.h"
+
+namespace xnor_hip {
+
+// n / d for 32-bit n by multiply-high and shifts; d is fixed on the host.
+struct FastDiv {
+    uint32_t mul, sh1, sh2, d;
+    __host__ static FastDiv make(uint32_t d) {
+        FastDiv f{0u, 0u, 0u, d};
+        if (d <= 1) return f;
+        uint32_t L = 0;
+        while ((1ull << L) < d) L++;
+        f.mul = (uint32_t)(((1ull << 32) * ((1ull << L) - d)) / d + 1);
+        f.sh1 = 1;
+        f.sh2 = L - 1;
+        return f;
+    }
+    __device__ __forceinline__ uint32_t div(uint32_t n) const {
+        uint32_t t = __umulhi(n, mul);
+        return (t + ((n - t) >> sh1)) >> sh2;
+    }
+};
+
+// Geometry shared by all kernels.  Device layouts:
+//   bin_src      uint32 [MB*IH*IW][XW]          word j, bit (31-b) = channel 32j+b has its
+//                                               sign bit clear; channels >= IC are 0
+//   bin_weights  uint32 [OCB][KH*KW][XW][Q]     same bit order; channels >= IC and
+//                                               filters >= OC are all ones
+//   alpha        float  [OC]
+//   a            float  [MB*IH*IW]
+//   k            float  [MB*OH*OW]
+//   op count     int32  [OH*OW]
+struct Geometry {
+    int mb, ic, ih, iw, oc, oh, ow, kh, kw, sh, sw, ph, pw;
+    int src_fmt, w_fmt, dst_fmt;
+    int xw;       // 32-bit words per pixel = ceil(ic/32)
+    int q;        // filters per wave in the convolution kernel
+    int ocb;      // ceil(oc/q)
+    int ihw, ohw; // ih*iw, oh*ow
+    uint32_t npix_in, npix_out; // mb*ihw, mb*ohw
+    FastDiv div_ihw, div_iw, div_ohw, div_ow;
+};
+
+struct State {
+    Geometry g;
+    hipStream_t stream = nullptr;
+    // staging buffers for host-side user tensors (allocated on first use)
+    void *stage_src = nullptr, *stage_weights = nullptr, *stage_dst = nullptr;
+    // One-shot hand-over from binarize_data to calculate_k: binarize_data reads the
+    // input anyway and also leaves mean|x| in res[a]; calculate_k may then skip its own
+    // pass over the input when it is called next with the same src and a buffers.
+    const void *a_ready_src = nullptr;
+    const void *a_ready_buf = nullptr;
+    bool verbose = false;
+};
+
+inline State *state_of(const xnor_nn_convolution_t *c) {
+    return reinterpret_cast<State *>(c->state);
+}
+
+// Kernel launchers (one per stage); each returns the hipError_t of the launch.
+hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
+        float *a_or_null, hipStream_t s);
+hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s);
+hipError_t launch_box_filter(const Geometry &g, const float *a, float *k, hipStream_t s);
+hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *bits,
+        float *alpha, int32_t *opc, hipStream_t s);
+hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
+        const uint32_t *wbits, const float *alpha, const float *k, const int32_t *opc,
+        float *dst, int32_t *popc_or_null, hipStream_t s);
+hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
+        hipStream_t s);
+const char *convolution_kernel_name(const Geometry &g);
+const char *binarize_kernel_name(const Geometry &g);
+
+int pick_q(int oc, int xw);
+
+} // namespace xnor_hip
