@@ -73,6 +73,11 @@ xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
 int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage,
         char *buf, size_t buf_bytes);
 
+/* Compute units and peak engine clock (kHz) of the current HIP device, as the runtime
+ * reports them; the figures the VALU roofline of the convolution kernel is priced with.
+ * The reference's counterpart is its CPUID probe (reference src/utils/cpuid.hpp:119-168). */
+xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz);
+
 #ifdef __cplusplus
 }
 #endif

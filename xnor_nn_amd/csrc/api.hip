@@ -432,6 +432,19 @@ xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
     return run_convolution(c, res, popc, true);
 }
 
+xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz) {
+    int dev = 0, cus = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess
+            || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess
+            || hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return xnor_nn_error_memory;
+    }
+    if (compute_units) *compute_units = cus;
+    if (clock_khz) *clock_khz = khz;
+    return xnor_nn_success;
+}
+
 int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage, char *buf,
         size_t buf_bytes) {
     if (!bcast_descriptor(c) || !buf || buf_bytes == 0) return 0;
