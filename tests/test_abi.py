@@ -1,0 +1,170 @@
+"""The C-ABI boundary without a GPU: the library loads, exports every function that
+include/*.h declares, the descriptor has the layout a C compiler gives it, and the host-only
+entry points behave like the reference's."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+from xnor_nn_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+
+
+def declared_functions():
+    names = set()
+    for header in ("xnor_nn.h", "xnor_nn_hip.h"):
+        text = open(os.path.join(INCLUDE, header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(xnor_nn_\w+)\s*\(", text))
+    return sorted(names)
+
+
+def test_every_declared_symbol_is_exported():
+    lib = C.CDLL(capi.library_path())
+    names = declared_functions()
+    assert len(names) >= 16
+    for name in names:
+        assert hasattr(lib, name), name
+    # and the ctypes tables cover exactly the declared set
+    assert set(names) == set(capi.CORE_SYMBOLS) | set(capi.HIP_SYMBOLS)
+
+
+def test_descriptor_layout_matches_a_c_compiler(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "xnor_nn.h"
+#include "xnor_nn_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(xnor_nn_convolution_t),
+        offsetof(xnor_nn_convolution_t, mb), offsetof(xnor_nn_convolution_t, src_format),
+        offsetof(xnor_nn_convolution_t, resource_size),
+        offsetof(xnor_nn_convolution_t, binarize_weights),
+        offsetof(xnor_nn_convolution_t, forward), offsetof(xnor_nn_convolution_t, state),
+        sizeof(xnor_nn_resources_t));
+    printf("%d %d %d %d %d %d\n", xnor_nn_unimplemented, xnor_nn_algorithm_bcast,
+        xnor_nn_resource_operations_count, xnor_nn_resource_number,
+        xnor_nn_weights_format_hwio, xnor_nn_operation_calculate_k);
+    return 0;
+}''')
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Werror", "-I", INCLUDE,
+                           str(src), "-o", str(exe)])
+    out = subprocess.check_output([str(exe)]).decode().split()
+    D = capi.ConvolutionDesc
+    want = [C.sizeof(D), D.mb.offset, D.src_format.offset, D.resource_size.offset,
+            D.binarize_weights.offset, D.forward.offset, D.state.offset,
+            C.sizeof(capi.Resources)]
+    assert [int(v) for v in out[:8]] == want
+    assert [int(v) for v in out[8:]] == [3, 1, 8, 9, 3, 3]
+
+
+def test_cpp_wrapper_header_compiles(tmp_path):
+    src = tmp_path / "wrap.cpp"
+    src.write_text('#include "xnor_nn.hpp"\n'
+                   'int use(const void *w) { xnor_nn::Convolution c{xnor_nn_algorithm_bcast,'
+                   ' xnor_nn_data_format_nchw, xnor_nn_weights_format_oihw,'
+                   ' xnor_nn_data_format_nchw, 1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1, w};'
+                   ' return 0; }\n')
+    subprocess.check_call(["g++", "-std=c++14", "-Wall", "-Werror", "-fsyntax-only",
+                           "-I", INCLUDE, str(src)])
+
+
+def test_status_messages():
+    """reference src/status.cpp:3-15"""
+    lib = capi.load()
+    assert [capi.status_message(lib, s) for s in range(4)] == [
+        "success", "memory_error", "bad_input", "unimplemented"]
+
+
+def test_init_fills_descriptor_like_the_reference():
+    """reference src/common_convolution.cpp:9-63: every field set, oh AND ow from pw,
+    always success; plus this library's device buffer sizes."""
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    st = lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, capi.FMT_NCHW,
+                                      capi.FMT_OIHW, capi.FMT_NCHW,
+                                      4, 256, 96, 27, 27, 5, 5, 1, 1, 2, 2)
+    assert st == capi.SUCCESS
+    assert (c.mb, c.ic, c.ih, c.iw, c.oc, c.oh, c.ow) == (4, 96, 27, 27, 256, 27, 27)
+    assert (c.kh, c.kw, c.sh, c.sw, c.ph, c.pw) == (5, 5, 1, 1, 2, 2)
+    assert c.state and all((c.binarize_weights, c.binarize_data, c.calculate_k, c.forward))
+    assert c.resource_size[capi.RES_BIN_SRC] == 4 * 27 * 27 * 3 * 4
+    assert c.resource_size[capi.RES_BIN_WEIGHTS] == 16 * 25 * 3 * 16 * 4
+    assert c.resource_size[capi.RES_A] == c.resource_size[capi.RES_K] == 4 * 27 * 27 * 4
+    assert c.resource_size[capi.RES_ALPHA] == 256 * 4
+    assert c.resource_size[capi.RES_OPERATIONS_COUNT] == 27 * 27 * 4
+    # oh uses pw, not ph (reference src/common_convolution.cpp:16)
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+    assert not c.state
+    lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, 0, 2, 0,
+                                 1, 16, 8, 10, 10, 3, 3, 1, 1, 0, 1)
+    assert (c.oh, c.ow) == (10, 10)
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+    lib.xnor_nn_destroy_convolution(C.byref(c))  # idempotent
+
+
+def test_null_and_format_checks_of_the_executors():
+    """Same status codes as the reference for missing slots
+    (reference src/bcast_binarize_data.cpp:15-19, src/bcast_calculate_k.cpp:15-20,
+    src/bcast_binarize_weights.cpp:15-21, src/default/bcast_convolution_default.cpp:25-33)
+    and unknown formats (reference src/bcast_binarize_data.cpp:36-38).  No GPU needed: the
+    checks come before any device work."""
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, capi.FMT_NCHW,
+                                 capi.FMT_OIHW, capi.FMT_NCHW, 1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1)
+    res = capi.Resources()
+    for stage in ("binarize_data", "calculate_k", "binarize_weights", "forward"):
+        assert getattr(c, stage)(C.byref(c), res) == capi.ERROR_INVALID_INPUT, stage
+    lib.xnor_nn_free_resources(res)  # safe on a zeroed table
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+
+    dummy = (C.c_float * 4)()
+    for i in range(capi.RES_NUMBER):
+        res[i] = C.addressof(dummy)
+    lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, 7, 9, 11,
+                                 1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1)
+    for stage in ("binarize_data", "calculate_k", "binarize_weights", "forward"):
+        assert getattr(c, stage)(C.byref(c), res) == capi.UNIMPLEMENTED, stage
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+
+
+def test_reference_algorithm_has_no_gpu_path():
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    st = lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_REFERENCE, 0, 2, 0,
+                                      1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1)
+    assert st == capi.SUCCESS and not c.state
+    res = capi.Resources()
+    assert c.forward(C.byref(c), res) == capi.UNIMPLEMENTED
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+
+
+def test_package_does_not_touch_the_oracle():
+    """The oracle is test infrastructure: nothing under xnor_nn_amd/ may name it."""
+    pkg = os.path.join(ROOT, "xnor_nn_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(base, f)
+
+
+@pytest.mark.skipif(not os.path.isdir("/root/reference/example"),
+                    reason="upstream sources not mounted")
+@pytest.mark.parametrize("name,cc", [("simple_convolution.c", "gcc"),
+                                     ("simple_convolution.cpp", "g++")])
+def test_upstream_examples_compile_and_link_unchanged(tmp_path, name, cc):
+    """The reference's own example programs (reference example/simple_convolution.c,
+    .cpp) build against include/ and link to libxnor_nn.so without edits."""
+    exe = tmp_path / "example"
+    libdir = os.path.dirname(capi.library_path())
+    subprocess.check_call([cc, "-I", INCLUDE, os.path.join("/root/reference/example", name),
+                           "-L", libdir, "-lxnor_nn", "-Wl,-rpath," + libdir,
+                           "-Wl,-rpath-link,/opt/rocm/lib", "-o", str(exe)])

@@ -1,0 +1,58 @@
+"""The C oracle against the REAL upstream library (oracle/_ref, built by
+`make -C oracle ref` where the upstream sources are mounted): every tensor bit for bit.
+Skipped when that library has not been built."""
+import numpy as np
+import pytest
+
+import shapes
+from util import oracle_shape
+from xnor_nn_amd import capi, synth
+
+KEYS = ("bin_src", "bin_weights", "a", "k", "alpha", "opc", "dst")
+
+
+def same_bytes(a, b):
+    return a.size * a.itemsize == b.size * b.itemsize and np.array_equal(
+        np.ascontiguousarray(a).view(np.uint8).ravel(),
+        np.ascontiguousarray(b).view(np.uint8).ravel())
+
+
+@pytest.mark.parametrize("t", shapes.COMPARE_WITH_REFERENCE, ids=shapes.shape_id)
+def test_reference_test_matrix(oracle, reflib, t):
+    d = shapes.as_dims(t)
+    x = synth.reference_test_src(d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.reference_test_weights(d["oc"], d["ic"], d["kh"], d["kw"])
+    mine = oracle.forward(oracle_shape(oracle, d), x, w)
+    ref = reflib.forward(d, x, w)
+    keys = KEYS if ref.get("bcast_applicable") else ("a", "k", "alpha", "dst")
+    for key in keys:
+        assert same_bytes(mine[key], ref[key]), key
+    # the upstream float algorithm (its own test oracle) agrees to its tolerance of 1e-3
+    alg = reflib.forward(d, x, w, algorithm=capi.ALGORITHM_REFERENCE)
+    assert np.allclose(mine["dst"], alg["dst"], atol=1e-3, rtol=0)
+
+
+@pytest.mark.parametrize("name,mb", [
+    ("alexnet_conv4_mb1", None), ("alexnet_conv4_mb256", 8), ("alexnet_conv2_mb128", 2),
+    ("resnet_3x3_mb64", 1), ("vgg_512_mb32", 2)])
+def test_workloads(oracle, reflib, name, mb):
+    d, x, w = synth.make_workload(name, mb)
+    mine = oracle.forward(oracle_shape(oracle, d), x, w)
+    ref = reflib.forward(d, x, w)
+    for key in KEYS:
+        assert same_bytes(mine[key], ref[key]), key
+
+
+def test_negative_zero_differs_between_upstream_algorithms(oracle, reflib):
+    """bcast takes the IEEE sign bit, the upstream float algorithm tests >= 0
+    (reference src/reference_convolution.cpp:102-103): they differ on -0.0 only, and the
+    oracle follows bcast."""
+    d = dict(mb=1, ic=16, oc=16, ih=4, iw=4, kh=3, kw=3, sh=1, sw=1, ph=1, pw=1)
+    x = synth.normal(3, 16 * 16).reshape(1, 16, 4, 4)
+    x[0, :, 1, 1] = -0.0
+    w = synth.normal(4, 16 * 16 * 9, 0.05).reshape(16, 16, 3, 3)
+    mine = oracle.forward(oracle_shape(oracle, d), x, w)
+    ref = reflib.forward(d, x, w)
+    assert same_bytes(mine["dst"], ref["dst"])
+    alg = reflib.forward(d, x, w, algorithm=capi.ALGORITHM_REFERENCE)
+    assert not np.allclose(mine["dst"], alg["dst"], atol=1e-3, rtol=0)
