@@ -96,7 +96,13 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="alexnet_conv4_mb256")
+    ap.add_argument("--mb", type=int, default=None,
+                    help="override the batch size of the workload (experiments only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="after the timed region, run one plain device-to-device copy of "
+                         "this many MiB (a kernel of known traffic to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings with)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: every image of the batch is independent, so "
@@ -115,7 +121,7 @@ def main():
         sys.exit("cannot query the HIP device")
     cus, clk_hz = c_cus.value, c_khz.value * 1e3
 
-    d, x, w = synth.make_workload(args.workload)
+    d, x, w = synth.make_workload(args.workload, args.mb)
     wf = work_figures(d)
     xt = torch.from_numpy(x).to(dev)
     wt = torch.from_numpy(w).to(dev)
@@ -200,6 +206,14 @@ def main():
         "device": {"name": props.name, "cus": cus, "clock_ghz": clk_hz / 1e9},
     }
     conv.close()
+    if args.copy_calibration_mib:
+        n = args.copy_calibration_mib * (1 << 20) // 4
+        src_buf = torch.ones(n, dtype=torch.float32, device=dev)
+        dst_buf = torch.empty_like(src_buf)
+        torch.cuda.synchronize()
+        dst_buf.copy_(src_buf)
+        torch.cuda.synchronize()
+        result["copy_calibration_bytes_each_way"] = n * 4
     if not args.no_cpu:
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         cb = cpu_baseline(d, x, w, threads)

@@ -5,6 +5,8 @@
 // src/bcast_calculate_k.cpp:42-85.  Both float reductions are evaluated in exactly the
 // reference's order with separately rounded products and sums (no FMA contraction), so
 // a and k come out bit-identical to the CPU library.
+#include <cstdlib>
+
 #include "plan.hpp"
 
 namespace xnor_hip {
@@ -22,30 +24,40 @@ __device__ __forceinline__ uint32_t top_bits(int n) {
 }
 
 // NCHW input.  One workgroup = 64 consecutive pixels of the flattened (mb, ih, iw) index;
-// wave w of the group owns the 32-channel slices w, w+NW, ... of those pixels.  A lane is
-// a pixel, so every load instruction reads 64 consecutive floats of one channel plane.
-// All 32 loads of a slice are issued before the first use.  Sign bits are shifted into
-// the lane's word with one funnel shift per element (a ballot would produce
-// pixel-major masks of one channel, i.e. the transpose of what is stored).
+// wave w of the group owns S consecutive 32-channel slices per round (slices
+// (r*NW + w)*S .. +S-1 in round r).  A lane is a pixel, so every load instruction reads 64
+// consecutive floats of one channel plane.  All 32*S loads of a wave are issued before
+// the first use.  Sign bits are shifted into the lane's word with one funnel shift per
+// element (a ballot would produce pixel-major masks of one channel, i.e. the transpose
+// of what is stored).
 //
-// mean|x| must be summed over channels in order.  The slices therefore hand the running
-// sum from wave to wave through LDS: slice s adds its 32 terms after slice s-1 has
-// published its result.  Loads of all slices are in flight during that chain.
+// mean|x| must be summed over channels in order.  The waves therefore hand the running
+// sum from one to the next through LDS: wave w adds its terms after wave w-1 has published
+// its result.  The loads of every wave are in flight during that chain.
 //
 // The packed words of the tile are staged in LDS and written as one contiguous run.
-template <bool WRITE_BITS, bool WRITE_A>
-__global__ __launch_bounds__(TILE * MAX_WAVES)
+//
+// Workgroup b works on tile (b % 8) * tiles_per_xcd + b / 8: workgroups are dealt to the
+// eight XCDs round-robin, so this gives each XCD one contiguous range of tiles and the
+// cache lines that straddle two neighbouring tiles (a channel plane is rarely a multiple
+// of 128 bytes) are fetched into one L2 instead of two.
+template <int S, bool WRITE_BITS, bool WRITE_A>
+__global__ __launch_bounds__(TILE * MAX_WAVES / S)
 void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
-        float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds) {
+        float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
+        const uint32_t ntiles, const uint32_t tiles_per_xcd) {
     extern __shared__ uint32_t lds[];
     float *chain = reinterpret_cast<float *>(lds); // [TILE]
     uint32_t *stage = lds + TILE;                  // [TILE][xw]
+
+    const uint32_t tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= ntiles) return;
 
     const int lane = threadIdx.x & (TILE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nw = blockDim.x >> 6;
 
-    const uint32_t p = blockIdx.x * TILE + lane;
+    const uint32_t p = tile * TILE + lane;
     const bool live = p < g.npix_in;
     const uint32_t pc = live ? p : g.npix_in - 1;
     const uint32_t img = g.div_ihw.div(pc);
@@ -55,36 +67,39 @@ void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bi
     if (wave == 0) chain[lane] = 0.f;
 
     for (int r = 0; r < rounds; r++) {
-        const int slice = r * nw + wave; // wave-uniform
-        const int c0 = slice * 32;
+        const int slice0 = (r * nw + wave) * S; // wave-uniform
+        const int c0 = slice0 * 32;
         const bool has = c0 < g.ic;
-        float t[32];
-        uint32_t neg = 0; // sign bits, first channel ends up in the MSB
+        float t[32 * S];
         if (has) {
             const float *col = base + (size_t)c0 * g.ihw;
-            float v[32];
-            if (c0 + 32 <= g.ic) {
+            if (c0 + 32 * S <= g.ic) {
 #pragma unroll
-                for (int i = 0; i < 32; i++) v[i] = col[(size_t)i * g.ihw];
+                for (int i = 0; i < 32 * S; i++) t[i] = col[(size_t)i * g.ihw];
             } else {
 #pragma unroll
-                for (int i = 0; i < 32; i++)
-                    v[i] = (c0 + i < g.ic) ? col[(size_t)i * g.ihw] : 0.f;
+                for (int i = 0; i < 32 * S; i++)
+                    t[i] = (c0 + i < g.ic) ? col[(size_t)i * g.ihw] : 0.f;
             }
 #pragma unroll
-            for (int i = 0; i < 32; i++) {
-                neg = __builtin_amdgcn_alignbit(neg, fbits(v[i]), 31);
-                t[i] = __fmul_rn(__builtin_fabsf(v[i]), inv_ic);
+            for (int sl = 0; sl < S; sl++) {
+                uint32_t neg = 0; // sign bits, first channel ends up in the MSB
+#pragma unroll
+                for (int i = 0; i < 32; i++) {
+                    neg = __builtin_amdgcn_alignbit(neg, fbits(t[32 * sl + i]), 31);
+                    t[32 * sl + i] = __fmul_rn(__builtin_fabsf(t[32 * sl + i]), inv_ic);
+                }
+                const int n = g.ic - (c0 + 32 * sl);
+                if (WRITE_BITS && n > 0)
+                    stage[lane * g.xw + slice0 + sl] = (~neg) & top_bits(n);
             }
-            const int n = min(32, g.ic - c0);
-            if (WRITE_BITS) stage[lane * g.xw + slice] = (~neg) & top_bits(n);
         }
-        // ordered hand-over of the running sum: slice s goes after slice s-1
+        // ordered hand-over of the running sum: wave s goes after wave s-1
         for (int s = 0; s < nw; s++) {
             if (s == wave && has) {
                 float acc = chain[lane];
 #pragma unroll
-                for (int i = 0; i < 32; i++) acc = __fadd_rn(acc, t[i]);
+                for (int i = 0; i < 32 * S; i++) acc = __fadd_rn(acc, t[i]);
                 chain[lane] = acc;
             }
             __syncthreads();
@@ -92,7 +107,7 @@ void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bi
     }
 
     const size_t tile_words = (size_t)TILE * g.xw;
-    const size_t first = (size_t)blockIdx.x * tile_words;
+    const size_t first = (size_t)tile * tile_words;
     const size_t total = (size_t)g.npix_in * g.xw;
     if (WRITE_BITS)
         for (uint32_t i = threadIdx.x; i < tile_words; i += blockDim.x)
@@ -158,7 +173,33 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
     k[p] = acc;
 }
 
-int data_waves(const Geometry &g) { return g.xw < MAX_WAVES ? g.xw : MAX_WAVES; }
+// Slices per wave.  Two slices per wave halve the waves of a workgroup but need over 100
+// VGPRs, which leaves no more workgroups resident than one slice per wave does; measured
+// equal or slower on MI355X, so one is used.
+int slices_per_wave(const Geometry &g) {
+    if (const char *e = getenv("XNOR_NN_HIP_BIN_S")) return atoi(e) == 2 ? 2 : 1;
+    (void)g;
+    return 1;
+}
+
+template <int S, bool WRITE_BITS, bool WRITE_A>
+void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
+    const int max_waves = MAX_WAVES / S;
+    const int need = (g.xw + S - 1) / S;
+    const int nw = need < max_waves ? need : max_waves;
+    const int rounds = (need + nw - 1) / nw;
+    const uint32_t ntiles = (g.npix_in + TILE - 1) / TILE;
+    const uint32_t per_xcd = (ntiles + 7) / 8;
+    const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
+    hipLaunchKernelGGL((binarize_nchw_kernel<S, WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
+            dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+}
+
+template <bool WRITE_BITS, bool WRITE_A>
+void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
+    if (slices_per_wave(g) == 2) launch_nchw<2, WRITE_BITS, WRITE_A>(g, x, bits, a, s);
+    else launch_nchw<1, WRITE_BITS, WRITE_A>(g, x, bits, a, s);
+}
 
 } // namespace
 
@@ -171,16 +212,8 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
         float *a_or_null, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
     if (g.src_fmt == xnor_nn_data_format_nchw) {
-        const int nw = data_waves(g);
-        const int rounds = (g.xw + nw - 1) / nw;
-        const unsigned blocks = (g.npix_in + TILE - 1) / TILE;
-        const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
-        if (a_or_null)
-            hipLaunchKernelGGL((binarize_nchw_kernel<true, true>), dim3(blocks),
-                    dim3(nw * TILE), lds, s, x, bits, a_or_null, g, inv_ic, rounds);
-        else
-            hipLaunchKernelGGL((binarize_nchw_kernel<true, false>), dim3(blocks),
-                    dim3(nw * TILE), lds, s, x, bits, a_or_null, g, inv_ic, rounds);
+        if (a_or_null) launch_nchw<true, true>(g, x, bits, a_or_null, s);
+        else launch_nchw<true, false>(g, x, bits, nullptr, s);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
         if (a_or_null)
@@ -196,12 +229,7 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
     if (g.src_fmt == xnor_nn_data_format_nchw) {
-        const int nw = data_waves(g);
-        const int rounds = (g.xw + nw - 1) / nw;
-        const unsigned blocks = (g.npix_in + TILE - 1) / TILE;
-        const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
-        hipLaunchKernelGGL((binarize_nchw_kernel<false, true>), dim3(blocks),
-                dim3(nw * TILE), lds, s, x, nullptr, a, g, inv_ic, rounds);
+        launch_nchw<false, true>(g, x, nullptr, a, s);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
         hipLaunchKernelGGL((binarize_generic_kernel<false, true>), dim3(blocks), dim3(256),
