@@ -131,6 +131,11 @@ xnor_nn_status_t exec_binarize_weights(const xnor_nn_convolution_t *c,
                 static_cast<int32_t *>(res[xnor_nn_resource_operations_count]), st->stream)
             != hipSuccess)
         return xnor_nn_error_memory;
+    if (st->g.use_mfma && launch_pack_weights_fp4(st->g, static_cast<const float *>(w),
+                reinterpret_cast<uint32_t *>(static_cast<char *>(
+                        res[xnor_nn_resource_bin_weights]) + st->g.wfrag_offset), st->stream)
+            != hipSuccess)
+        return xnor_nn_error_memory;
     return xnor_nn_success;
 }
 
@@ -147,8 +152,12 @@ xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resourc
         out = st->stage_dst;
     }
     if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
-    if (launch_convolution(st->g, static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]),
-                static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]),
+    const uint32_t *wbits = static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]);
+    if (st->g.use_mfma)
+        wbits = reinterpret_cast<const uint32_t *>(
+                static_cast<const char *>(res[xnor_nn_resource_bin_weights]) + st->g.wfrag_offset);
+    if ((st->g.use_mfma ? launch_convolution_mfma : launch_convolution)(st->g,
+                static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]), wbits,
                 static_cast<const float *>(res[xnor_nn_resource_alpha]),
                 static_cast<const float *>(res[xnor_nn_resource_k]),
                 static_cast<const int32_t *>(res[xnor_nn_resource_operations_count]),
@@ -261,7 +270,11 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
     // Byte sizes of the device buffers (the reference's are host sizes of its CPU layout,
     // src/bcast_convolution.cpp:72-82).
     c->resource_size[xnor_nn_resource_bin_src] = (size_t)g.npix_in * g.xw * 4;
-    c->resource_size[xnor_nn_resource_bin_weights] = (size_t)g.ocb * kh * kw * g.xw * g.q * 4;
+    const size_t bit_bytes = (size_t)g.ocb * kh * kw * g.xw * g.q * 4;
+    g.use_mfma = mfma_applicable(g) ? 1 : 0;
+    g.wfrag_offset = (bit_bytes + 255) / 256 * 256;
+    c->resource_size[xnor_nn_resource_bin_weights] =
+        g.use_mfma ? g.wfrag_offset + mfma_weight_bytes(g) : bit_bytes;
     c->resource_size[xnor_nn_resource_a] = (size_t)g.npix_in * 4;
     c->resource_size[xnor_nn_resource_k] = (size_t)g.npix_out * 4;
     c->resource_size[xnor_nn_resource_alpha] = (size_t)oc * 4;

@@ -1,0 +1,342 @@
+// Stage 3 on the matrix cores: the same +-1 dot products as the XNOR/popcount kernel, as an
+// implicit GEMM in FP4 (E2M1 holds +1, -1 and 0 exactly; products are accumulated in FP32,
+// which is exact for |sum| < 2^24, so every accumulator equals 2*popc - n as an integer).
+// Semantics: reference src/default/bcast_convolution_default.cpp:60-105.
+//
+// Why FP4 MFMA rather than v_xnor/v_bcnt: one v_mfma_f32_32x32x64_f8f6f4 does 65536
+// multiply-accumulates in ~32 cycles per SIMD, the XNOR/popcount pair does 2048 in 8; the
+// measured ceilings on MI355X are 8.1 POP/s against 1.1 POP/s.  Out-of-bounds taps read a
+// row of FP4 zeros, which contributes nothing, so "skip the tap" needs no predication.
+//
+// Shape of the GEMM: C[oc][pixel] = sum over (tap, channel) W[oc][tap, channel] *
+// X[pixel shifted by tap][channel].  Filters are the A operand (rows), pixels the B
+// operand (columns): in the 32x32 accumulator layout a register then holds 32 consecutive
+// pixels of one filter, i.e. 128 contiguous bytes of the NCHW output.
+//
+// Workgroup = 128 consecutive output pixels x 128 filters, four waves of 64 x 64.
+//   * X: the packed sign bits of every input pixel the tile touches are expanded to FP4
+//     once and kept in LDS, one row per input pixel (channel-major, 16 spare bytes per row
+//     so that the 32 rows a fragment load touches spread over all banks).  A tap is a row
+//     offset; invalid taps point at a zero row.
+//   * W: pre-packed on the weight stage in fragment order (1 KB per 32 filters x 64
+//     channels), loaded straight into registers one tap ahead of use.
+#include <cstdlib>
+
+#include "plan.hpp"
+
+namespace xnor_hip {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int MT = 128;       // output pixels per workgroup
+constexpr int NT = 128;       // filters per workgroup
+constexpr int ROW_PAD = 16;   // spare bytes per LDS row
+constexpr int TABLE_BYTES = 1024;
+constexpr int LDS_LIMIT = 64 * 1024;
+
+// First and last input pixel (flattened index) that the tile of MT output pixels starting
+// at tile*MT can touch with an in-bounds tap, for stride 1: from the start of the first
+// input row of its first pixel to the end of the last input row of its last pixel.
+__host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, int &lo, int &hi) {
+    const uint32_t p_first = tile * MT;
+    uint32_t p_last = p_first + MT;
+    if (p_last > g.npix_out) p_last = g.npix_out;
+    p_last -= 1;
+    const uint32_t i0 = p_first / g.ohw, i1 = p_last / g.ohw;
+    const int oh0 = (int)((p_first - i0 * g.ohw) / g.ow);
+    const int oh1 = (int)((p_last - i1 * g.ohw) / g.ow);
+    int r0 = oh0 - g.ph, r1 = oh1 - g.ph + g.kh - 1;
+    if (r0 < 0) r0 = 0;
+    if (r0 > g.ih - 1) r0 = g.ih - 1;
+    if (r1 > g.ih - 1) r1 = g.ih - 1;
+    if (r1 < 0) r1 = 0;
+    lo = (int)(i0 * g.ihw) + r0 * g.iw;
+    hi = (int)(i1 * g.ihw) + r1 * g.iw + g.iw - 1;
+    if (hi < lo) hi = lo;
+}
+
+__device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c) {
+    const v8i a8 = {a.x, a.y, a.z, a.w, 0, 0, 0, 0};
+    const v8i b8 = {b.x, b.y, b.z, b.w, 0, 0, 0, 0};
+    // cbsz = blgp = 4: both operands FP4 (E2M1); scales 0x7f = 2^0
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, 0, 0x7f7f7f7f, 0,
+            0x7f7f7f7f);
+}
+
+// FP4 codes of eight channels from one byte of packed sign bits (bit 7 = first channel,
+// set = sign bit clear = +1): nibble i = channel i, +1 -> 0x2, -1 -> 0xA.
+__device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
+    uint32_t out = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        out |= (((byte >> (7 - i)) & 1u) ? 0x2u : 0xAu) << (4 * i);
+    return out;
+}
+
+// KS = 64-channel steps per tap = ceil(IC / 64).
+template <int KS, bool RAW>
+__global__ __launch_bounds__(256, 2)
+void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
+        const float *__restrict__ alpha, const float *__restrict__ kplane,
+        const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
+        const Geometry g, const int max_rows, const int oc_chunks) {
+    extern __shared__ unsigned char smem[];
+    uint32_t *table = reinterpret_cast<uint32_t *>(smem);
+    unsigned char *rows = smem + TABLE_BYTES; // row 0 is all zero, staged rows follow
+    constexpr int ROW_BYTES = KS * 32 + ROW_PAD;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tile = blockIdx.x / oc_chunks;
+    const int chunk = blockIdx.x - tile * oc_chunks;
+    const int taps = g.kh * g.kw;
+
+    // ---- which input pixels does the tile touch (stride 1) ----------------------------
+    const uint32_t p_first = tile * MT;
+    int lo, hi;
+    tile_span(g, tile, lo, hi);
+    const int nrows = min(hi - lo + 1, max_rows);
+
+    // ---- LDS: lookup table, zero row, FP4 rows -------------------------------------------
+    table[tid] = fp4_of_byte(tid);
+    for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < nrows * KS * 2; i += 256) {
+        const int r = i / (KS * 2), j = i - r * (KS * 2); // row, 32-channel word
+        v4i q = {0, 0, 0, 0};
+        if (j < g.xw) {
+            const uint32_t w = xbits[(size_t)(lo + r) * g.xw + j];
+            q.x = table[w >> 24];
+            q.y = table[(w >> 16) & 0xFF];
+            q.z = table[(w >> 8) & 0xFF];
+            q.w = table[w & 0xFF];
+        }
+        *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
+    }
+
+    // ---- this wave's 64 filters x 64 pixels -------------------------------------------------
+    const int oc_sub0 = chunk * (NT / 32) + (wave & 1) * 2; // first 32-filter block
+    const uint32_t p_wave = p_first + (wave >> 1) * 64;
+    bool live[2];
+    int in0[2], oh[2], ow[2]; // input index of tap (0,0) relative to lo; output coordinates
+    uint32_t pix[2], img[2], rem[2];
+#pragma unroll
+    for (int ps = 0; ps < 2; ps++) {
+        pix[ps] = p_wave + ps * 32 + (lane & 31);
+        live[ps] = pix[ps] < g.npix_out;
+        const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
+        img[ps] = g.div_ohw.div(pc);
+        rem[ps] = pc - img[ps] * g.ohw;
+        oh[ps] = (int)g.div_ow.div(rem[ps]);
+        ow[ps] = (int)rem[ps] - oh[ps] * g.ow;
+        in0[ps] = (int)(img[ps] * g.ihw) + (oh[ps] - g.ph) * g.iw + (ow[ps] - g.pw) - lo;
+    }
+    const int half_off = (lane >> 5) * 16;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int os = 0; os < 2; os++)
+#pragma unroll
+        for (int ps = 0; ps < 2; ps++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[os][ps][i] = 0.f;
+
+    // weight fragments: [32-filter block][tap][step][lane]
+    auto load_tap = [&](int t, v4i (&w)[KS][2]) {
+#pragma unroll
+        for (int os = 0; os < 2; os++) {
+            const v4i *src = wfrag + ((size_t)(oc_sub0 + os) * taps + t) * KS * 64 + lane;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) w[ks][os] = src[ks * 64];
+        }
+    };
+    auto compute_tap = [&](int t, const v4i (&w)[KS][2]) {
+        const int kh = t / g.kw, kw = t - kh * g.kw;
+        int addr[2];
+#pragma unroll
+        for (int ps = 0; ps < 2; ps++) {
+            const int ih = oh[ps] - g.ph + kh, iw = ow[ps] - g.pw + kw;
+            const int r = in0[ps] + kh * g.iw + kw;
+            const bool ok = live[ps] && (unsigned)ih < (unsigned)g.ih
+                && (unsigned)iw < (unsigned)g.iw && (unsigned)r < (unsigned)nrows;
+            addr[ps] = (ok ? (1 + r) * ROW_BYTES : 0) + half_off;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            v4i b[2];
+#pragma unroll
+            for (int ps = 0; ps < 2; ps++)
+                b[ps] = *reinterpret_cast<const v4i *>(rows + addr[ps] + ks * 32);
+#pragma unroll
+            for (int os = 0; os < 2; os++)
+#pragma unroll
+                for (int ps = 0; ps < 2; ps++)
+                    acc[os][ps] = mfma_fp4(w[ks][os], b[ps], acc[os][ps]);
+        }
+    };
+
+    v4i wa[KS][2], wb[KS][2];
+    load_tap(0, wa);
+    __syncthreads(); // FP4 rows are in place
+    for (int t = 0; t < taps; t += 2) {
+        if (t + 1 < taps) load_tap(t + 1, wb);
+        compute_tap(t, wa);
+        if (t + 1 < taps) {
+            if (t + 2 < taps) load_tap(t + 2, wa);
+            compute_tap(t + 1, wb);
+        }
+    }
+
+    // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
+    //      pixel lane%32 ------------------------------------------------------------------------
+#pragma unroll
+    for (int ps = 0; ps < 2; ps++) {
+        if (!live[ps]) continue;
+        const int n = opc[rem[ps]];
+        const float kv = RAW ? 0.f : kplane[pix[ps]];
+#pragma unroll
+        for (int os = 0; os < 2; os++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int oc = (oc_sub0 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4 + (i & 3);
+                if (oc >= g.oc) continue;
+                const float d = acc[os][ps][i]; // = 2*popc - n, exactly
+                if constexpr (RAW) {
+                    popc[((size_t)img[ps] * g.oc + oc) * g.ohw + rem[ps]] = ((int)d + n) / 2;
+                } else {
+                    // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
+                    const float v = __fmul_rn(__fmul_rn(d, alpha[oc]), kv);
+                    if (g.dst_fmt == xnor_nn_data_format_nchw)
+                        dst[((size_t)img[ps] * g.oc + oc) * g.ohw + rem[ps]] = v;
+                    else
+                        dst[(size_t)pix[ps] * g.oc + oc] = v;
+                }
+            }
+        }
+    }
+}
+
+// One thread per dword of the fragment layout [OC/32][tap][KS][lane][4 dwords]:
+// lane l of a fragment holds filter (l % 32) and channels (l / 32) * 32 .. +31 of the step,
+// eight channels per dword, low nibble first.  Channels >= IC and filters >= OC are FP4 zero.
+__global__ __launch_bounds__(256)
+void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__ frag,
+        const Geometry g, const int ks_n, const int oc_subs) {
+    const int taps = g.kh * g.kw;
+    const size_t total = (size_t)oc_subs * taps * ks_n * 64 * 4;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int dw = (int)(i & 3);
+    const int lane = (int)((i >> 2) & 63);
+    const size_t f = i >> 8; // fragment index
+    const int ks = (int)(f % ks_n);
+    const int tap = (int)((f / ks_n) % taps);
+    const int sub = (int)(f / ((size_t)ks_n * taps));
+    const int oc = sub * 32 + (lane & 31);
+    const int c0 = ks * 64 + (lane >> 5) * 32 + dw * 8;
+    const int kh = tap / g.kw, kw = tap % g.kw;
+    uint32_t out = 0;
+    for (int n = 0; n < 8; n++) {
+        const int c = c0 + n;
+        if (oc < g.oc && c < g.ic) {
+            const size_t at = g.w_fmt == xnor_nn_weights_format_oihw
+                ? (((size_t)oc * g.ic + c) * g.kh + kh) * g.kw + kw
+                : (((size_t)kh * g.kw + kw) * g.ic + c) * g.oc + oc;
+            out |= ((__float_as_uint(w[at]) >> 31) ? 0xAu : 0x2u) << (4 * n);
+        }
+    }
+    frag[i] = out;
+}
+
+int steps_per_tap(const Geometry &g) { return (g.ic + 63) / 64; }
+int oc_subblocks(const Geometry &g) { return ((g.oc + NT - 1) / NT) * (NT / 32); }
+
+// Largest number of input pixels any tile touches.  The offset of a tile within its image
+// repeats after at most OHW tiles, so that many (plus the last, possibly short, tile) are
+// enough to look at.
+int max_tile_rows(const Geometry &g) {
+    const uint32_t tiles = (g.npix_out + MT - 1) / MT;
+    const uint32_t look = tiles < (uint32_t)g.ohw + 1 ? tiles : (uint32_t)g.ohw + 1;
+    int most = 1;
+    for (uint32_t t = 0; t < look; t++) {
+        int lo, hi;
+        tile_span(g, t, lo, hi);
+        if (hi - lo + 1 > most) most = hi - lo + 1;
+    }
+    int lo, hi;
+    tile_span(g, tiles - 1, lo, hi);
+    if (hi - lo + 1 > most) most = hi - lo + 1;
+    return most;
+}
+
+size_t lds_bytes(const Geometry &g) {
+    return TABLE_BYTES + (size_t)(1 + max_tile_rows(g)) * (steps_per_tap(g) * 32 + ROW_PAD);
+}
+
+template <int KS>
+hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
+        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        hipStream_t s) {
+    const int chunks = (g.oc + NT - 1) / NT;
+    const uint32_t tiles = (g.npix_out + MT - 1) / MT;
+    const dim3 grid(tiles * chunks), block(256);
+    const int rows = max_tile_rows(g);
+    const size_t lds = lds_bytes(g);
+    const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
+    if (popc)
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, true>), grid, block, lds, s, xbits, wf,
+                alpha, k, opc, dst, popc, g, rows, chunks);
+    else
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, false>), grid, block, lds, s, xbits, wf,
+                alpha, k, opc, dst, popc, g, rows, chunks);
+    return hipGetLastError();
+}
+
+} // namespace
+
+// The matrix-core kernel covers stride-1 convolutions with up to 512 input channels whose
+// tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
+// XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
+bool mfma_applicable(const Geometry &g) {
+    if (const char *e = getenv("XNOR_NN_HIP_CONV"))
+        if (e[0] == 'v') return false;
+    if (g.sh != 1 || g.sw != 1) return false;
+    if (steps_per_tap(g) > 8) return false;
+    if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return false;
+    return lds_bytes(g) <= (size_t)LDS_LIMIT;
+}
+
+size_t mfma_weight_bytes(const Geometry &g) {
+    return (size_t)oc_subblocks(g) * g.kh * g.kw * steps_per_tap(g) * 1024;
+}
+
+hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
+        hipStream_t s) {
+    const size_t dwords = mfma_weight_bytes(g) / 4;
+    hipLaunchKernelGGL(pack_weights_fp4_kernel, dim3((unsigned)((dwords + 255) / 256)),
+            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g));
+    return hipGetLastError();
+}
+
+hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
+        const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
+        float *dst, int32_t *popc, hipStream_t s) {
+    switch (steps_per_tap(g)) {
+    case 1: return launch_mfma<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 2: return launch_mfma<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 3: return launch_mfma<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 4: return launch_mfma<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 5: return launch_mfma<5>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 6: return launch_mfma<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 7: return launch_mfma<7>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 8: return launch_mfma<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+} // namespace xnor_hip

@@ -37,7 +37,9 @@ struct FastDiv {
 //   bin_src      uint32 [MB*IH*IW][XW]          word j, bit (31-b) = channel 32j+b has its
 //                                               sign bit clear; channels >= IC are 0
 //   bin_weights  uint32 [OCB][KH*KW][XW][Q]     same bit order; channels >= IC and
-//                                               filters >= OC are all ones
+//                                               filters >= OC are all ones; followed (at
+//                                               wfrag_offset) by the same signs as FP4
+//                                               matrix-core fragments when use_mfma is set
 //   alpha        float  [OC]
 //   a            float  [MB*IH*IW]
 //   k            float  [MB*OH*OW]
@@ -50,6 +52,8 @@ struct Geometry {
     int ocb;      // ceil(oc/q)
     int ihw, ohw; // ih*iw, oh*ow
     uint32_t npix_in, npix_out; // mb*ihw, mb*ohw
+    int use_mfma;               // 1: stage 3 runs the FP4 matrix-core kernel
+    size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
 
@@ -82,6 +86,13 @@ hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         float *dst, int32_t *popc_or_null, hipStream_t s);
 hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
         hipStream_t s);
+bool mfma_applicable(const Geometry &g);
+size_t mfma_weight_bytes(const Geometry &g);
+hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
+        hipStream_t s);
+hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
+        const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
+        float *dst, int32_t *popc_or_null, hipStream_t s);
 const char *convolution_kernel_name(const Geometry &g);
 const char *binarize_kernel_name(const Geometry &g);
 
