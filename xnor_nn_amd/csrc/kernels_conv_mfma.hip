@@ -21,6 +21,7 @@
 //   * W: pre-packed on the weight stage in fragment order (1 KB per 32 filters x 64
 //     channels), loaded straight into registers one tap ahead of use.
 #include <cstdlib>
+#include <type_traits>
 
 #include "plan.hpp"
 
@@ -36,6 +37,7 @@ constexpr int MT = 128;       // output pixels per workgroup
 constexpr int NT = 128;       // filters per workgroup
 constexpr int ROW_PAD = 16;   // spare bytes per LDS row
 constexpr int TABLE_BYTES = 1024;
+constexpr int ALPHA_BYTES = NT * 4;
 constexpr int LDS_LIMIT = 64 * 1024;
 
 // First and last input pixel (flattened index) that the tile of MT output pixels starting
@@ -86,7 +88,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const Geometry g, const int max_rows, const int oc_chunks) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
-    unsigned char *rows = smem + TABLE_BYTES; // row 0 is all zero, staged rows follow
+    float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
+    unsigned char *rows = smem + TABLE_BYTES + ALPHA_BYTES; // row 0 is zero, then the tile
     constexpr int ROW_BYTES = KS * 32 + ROW_PAD;
 
     const int tid = threadIdx.x;
@@ -102,21 +105,42 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     tile_span(g, tile, lo, hi);
     const int nrows = min(hi - lo + 1, max_rows);
 
-    // ---- LDS: lookup table, zero row, FP4 rows -------------------------------------------
+    // ---- LDS: lookup table, zero row, this workgroup's alphas, FP4 rows ----------------------
     table[tid] = fp4_of_byte(tid);
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
+    if (tid < NT) {
+        const int oc = chunk * NT + tid;
+        alpha_lds[tid] = oc < g.oc ? alpha[oc] : 0.f;
+    }
     __syncthreads();
-    for (int i = tid; i < nrows * KS * 2; i += 256) {
-        const int r = i / (KS * 2), j = i - r * (KS * 2); // row, 32-channel word
-        v4i q = {0, 0, 0, 0};
-        if (j < g.xw) {
-            const uint32_t w = xbits[(size_t)(lo + r) * g.xw + j];
-            q.x = table[w >> 24];
-            q.y = table[(w >> 16) & 0xFF];
-            q.z = table[(w >> 8) & 0xFF];
-            q.w = table[w & 0xFF];
+    // The rows of the tile are contiguous in the packed input: item i is word i of that
+    // run.  Four loads per thread are issued before the first is expanded.  Words past
+    // ceil(IC/32) of a row are left as they are: the matching weights are FP4 zeros and
+    // FP4 has no NaN or infinity, so whatever LDS holds there contributes nothing.
+    {
+        const int nitems = nrows * g.xw;
+        const uint32_t *run = xbits + (size_t)lo * g.xw;
+        for (int base = 0; base < nitems; base += 4 * 256) {
+            uint32_t w[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = base + u * 256 + tid;
+                w[u] = i < nitems ? run[i] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = base + u * 256 + tid;
+                if (i < nitems) {
+                    const int r = i / g.xw, j = i - r * g.xw; // row, 32-channel word
+                    v4i q;
+                    q.x = table[w[u] >> 24];
+                    q.y = table[(w[u] >> 16) & 0xFF];
+                    q.z = table[(w[u] >> 8) & 0xFF];
+                    q.w = table[w[u] & 0xFF];
+                    *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
+                }
+            }
         }
-        *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
     }
 
     // ---- this wave's 64 filters x 64 pixels -------------------------------------------------
@@ -180,45 +204,56 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         }
     };
 
-    v4i wa[KS][2], wb[KS][2];
-    load_tap(0, wa);
+    // One tap ahead: the fragments of tap t+1 are requested before tap t is multiplied and
+    // only waited for (by the copy) after its 4*KS matrix instructions have been issued.
+    v4i wcur[KS][2], wnext[KS][2];
+    load_tap(0, wcur);
     __syncthreads(); // FP4 rows are in place
-    for (int t = 0; t < taps; t += 2) {
-        if (t + 1 < taps) load_tap(t + 1, wb);
-        compute_tap(t, wa);
-        if (t + 1 < taps) {
-            if (t + 2 < taps) load_tap(t + 2, wa);
-            compute_tap(t + 1, wb);
-        }
+    for (int t = 0; t < taps; t++) {
+        if (t + 1 < taps) load_tap(t + 1, wnext);
+        compute_tap(t, wcur);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int os = 0; os < 2; os++) wcur[ks][os] = wnext[ks][os];
     }
 
     // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
     //      pixel lane%32 ------------------------------------------------------------------------
+    auto store_tile = [&](auto check_filters) {
 #pragma unroll
-    for (int ps = 0; ps < 2; ps++) {
-        if (!live[ps]) continue;
-        const int n = opc[rem[ps]];
-        const float kv = RAW ? 0.f : kplane[pix[ps]];
+        for (int ps = 0; ps < 2; ps++) {
+            if (!live[ps]) continue;
+            const int n = opc[rem[ps]];
+            const float kv = RAW ? 0.f : kplane[pix[ps]];
+            const size_t nchw0 = ((size_t)img[ps] * g.oc) * g.ohw + rem[ps];
 #pragma unroll
-        for (int os = 0; os < 2; os++) {
+            for (int os = 0; os < 2; os++) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int oc = (oc_sub0 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4 + (i & 3);
-                if (oc >= g.oc) continue;
-                const float d = acc[os][ps][i]; // = 2*popc - n, exactly
-                if constexpr (RAW) {
-                    popc[((size_t)img[ps] * g.oc + oc) * g.ohw + rem[ps]] = ((int)d + n) / 2;
-                } else {
-                    // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
-                    const float v = __fmul_rn(__fmul_rn(d, alpha[oc]), kv);
-                    if (g.dst_fmt == xnor_nn_data_format_nchw)
-                        dst[((size_t)img[ps] * g.oc + oc) * g.ohw + rem[ps]] = v;
-                    else
-                        dst[(size_t)pix[ps] * g.oc + oc] = v;
+                for (int i = 0; i < 16; i++) {
+                    const int ocl = ((wave & 1) * 2 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4
+                        + (i & 3);
+                    const int oc = chunk * NT + ocl;
+                    if (decltype(check_filters)::value && oc >= g.oc) continue;
+                    const float d = acc[os][ps][i]; // = 2*popc - n, exactly
+                    if constexpr (RAW) {
+                        popc[nchw0 + (size_t)oc * g.ohw] = ((int)d + n) / 2;
+                    } else {
+                        // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
+                        const float v = __fmul_rn(__fmul_rn(d, alpha_lds[ocl]), kv);
+                        if (g.dst_fmt == xnor_nn_data_format_nchw)
+                            dst[nchw0 + (size_t)oc * g.ohw] = v;
+                        else
+                            dst[(size_t)pix[ps] * g.oc + oc] = v;
+                    }
                 }
             }
         }
-    }
+    };
+    if ((chunk + 1) * NT <= g.oc) // workgroup-uniform: every filter of the chunk exists
+        store_tile(std::false_type{});
+    else
+        store_tile(std::true_type{});
 }
 
 // One thread per dword of the fragment layout [OC/32][tap][KS][lane][4 dwords]:
@@ -275,7 +310,7 @@ int max_tile_rows(const Geometry &g) {
 }
 
 size_t lds_bytes(const Geometry &g) {
-    return TABLE_BYTES + (size_t)(1 + max_tile_rows(g)) * (steps_per_tap(g) * 32 + ROW_PAD);
+    return TABLE_BYTES + ALPHA_BYTES + (size_t)(1 + max_tile_rows(g)) * (steps_per_tap(g) * 32 + ROW_PAD);
 }
 
 template <int KS>
