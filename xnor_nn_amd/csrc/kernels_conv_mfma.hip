@@ -69,6 +69,24 @@ __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c)
             0x7f7f7f7f);
 }
 
+// Weight fragments are fetched with hand-issued loads and hand-placed waits: left to
+// itself the compiler hoists the loads of the next tap to the top of the current one and
+// then waits for them before the first matrix instruction.
+//   * load_frag_async only starts the load; the register holds the data once a later
+//     wait_loads_after() has run.
+//   * wait_loads_after() is "s_waitcnt vmcnt(0)" carrying the four accumulator tiles as
+//     read-write operands.  That data dependence orders it behind the matrix instructions
+//     issued before it and ahead of those that follow, which are the ones that consume
+//     the awaited fragments.  The fragments themselves are deliberately not operands: a
+//     read-write operand lets the compiler copy the register on the way in, and a copy of
+//     a register whose load is still in flight copies stale data.
+__device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src));
+}
+__device__ __forceinline__ void wait_loads_after(v16f &a, v16f &b, v16f &c, v16f &d) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+
 // FP4 codes of eight channels from one byte of packed sign bits (bit 7 = first channel,
 // set = sign bit clear = +1): nibble i = channel i, +1 -> 0x2, -1 -> 0xA.
 __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
@@ -170,16 +188,22 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[os][ps][i] = 0.f;
 
-    // weight fragments: [32-filter block][tap][step][lane]
-    auto load_tap = [&](int t, v4i (&w)[KS][2]) {
+    // Weight fragments: [32-filter block][tap][step][lane], two register sets used in turn.
+    // The fragments of tap t+1 are requested before tap t is multiplied and awaited after
+    // its 4*KS matrix instructions; every request is awaited before the loop edge, so no
+    // register with a load in flight is live across it.
+    const v4i *wsrc[2];
 #pragma unroll
-        for (int os = 0; os < 2; os++) {
-            const v4i *src = wfrag + ((size_t)(oc_sub0 + os) * taps + t) * KS * 64 + lane;
+    for (int os = 0; os < 2; os++)
+        wsrc[os] = wfrag + (size_t)(oc_sub0 + os) * taps * KS * 64 + lane;
+    auto request_tap = [&](int t, v4i (&w)[KS][2]) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) w[ks][os] = src[ks * 64];
-        }
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int os = 0; os < 2; os++)
+                load_frag_async(w[ks][os], wsrc[os] + ((size_t)t * KS + ks) * 64);
     };
-    auto compute_tap = [&](int t, const v4i (&w)[KS][2]) {
+    auto multiply_tap = [&](int t, const v4i (&w)[KS][2]) {
         const int kh = t / g.kw, kw = t - kh * g.kw;
         int addr[2];
 #pragma unroll
@@ -204,22 +228,22 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         }
     };
 
-    // One tap ahead: the fragments of tap t+1 are requested before tap t is multiplied and
-    // only waited for (by the copy) after its 4*KS matrix instructions have been issued.
-    v4i wcur[KS][2], wnext[KS][2];
-    load_tap(0, wcur);
+    v4i wa[KS][2], wb[KS][2];
+    request_tap(0, wa);
+    wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]);
     __syncthreads(); // FP4 rows are in place
-    for (int t = 0; t < taps; t++) {
-        if (t + 1 < taps) load_tap(t + 1, wnext);
-        compute_tap(t, wcur);
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-            for (int os = 0; os < 2; os++) wcur[ks][os] = wnext[ks][os];
+    for (int t = 0; t < taps; t += 2) {
+        const bool second = t + 1 < taps, third = t + 2 < taps;
+        if (second) request_tap(t + 1, wb);
+        multiply_tap(t, wa);
+        if (second) {
+            wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]); // wb has landed
+            if (third) request_tap(t + 2, wa);
+            multiply_tap(t + 1, wb);
+            if (third) wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]); // wa
+        }
     }
 
-    // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
-    //      pixel lane%32 ------------------------------------------------------------------------
     auto store_tile = [&](auto check_filters) {
 #pragma unroll
         for (int ps = 0; ps < 2; ps++) {
