@@ -150,6 +150,12 @@ def test_tensor_formats(oracle, fmts, t):
     (5, 64, 64, 5, 9, 1, 1, 1, 1, 0, 0),      # 1x1 filter
     (2, 16, 32, 8, 8, 3, 3, 1, 1, 0, 0),      # no padding
     (1, 24, 16, 12, 12, 7, 7, 3, 3, 3, 3),    # big filter, stride 3
+    (2, 160, 100, 9, 9, 3, 3, 1, 1, 1, 1),    # 3 channel steps of 64, ragged filter count
+    (2, 288, 300, 7, 7, 3, 3, 1, 1, 1, 1),    # 5 steps (run as 6), more than 256 filters
+    (1, 448, 70, 6, 6, 3, 3, 1, 1, 1, 1),     # 7 steps (run as 8)
+    (7, 64, 40, 10, 10, 3, 3, 1, 1, 2, 2),    # padding larger than the usual "same"
+    (2, 32, 64, 16, 16, 4, 4, 1, 1, 0, 0),    # even filter size, output smaller than input
+    (1, 640, 32, 5, 5, 3, 3, 1, 1, 1, 1),     # more than 512 channels: popcount kernel
 ], ids=shapes.shape_id)
 def test_edge_shapes(oracle, t):
     d = shapes.as_dims(t)
@@ -161,6 +167,27 @@ def test_edge_shapes(oracle, t):
         d["oc"], d["ic"], d["kh"], d["kw"])
     w.ravel()[::13] = -0.0
     run_and_compare(oracle, d, x, w)
+
+
+@pytest.mark.parametrize("ps", ["2", "3", "4"])
+def test_matrix_core_tile_sizes(oracle, gpu, monkeypatch, ps):
+    """Every tile size of the matrix-core kernel on a workload whose last tile is ragged."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_PS", ps)
+    d, x, w = synth.make_workload("alexnet_conv4_mb256", 5)
+    run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+    d, x, w = synth.make_workload("vgg_512_mb32", 1)
+    run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+
+
+def test_popcount_kernel_still_matches(oracle, gpu, monkeypatch):
+    """The XNOR/popcount kernel (the general fallback) on shapes the matrix-core kernel
+    would otherwise take."""
+    monkeypatch.setenv("XNOR_NN_HIP_CONV", "valu")
+    for name, mb in (("alexnet_conv4_mb256", 4), ("alexnet_conv2_mb128", 2)):
+        d, x, w = synth.make_workload(name, mb)
+        conv_name = make(d, w).kernel_name(0)
+        assert conv_name.startswith("conv_xnor_popc"), conv_name
+        run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
 
 
 def test_known_answer_forward_on_gpu():

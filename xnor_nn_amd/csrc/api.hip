@@ -271,7 +271,17 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
     // src/bcast_convolution.cpp:72-82).
     c->resource_size[xnor_nn_resource_bin_src] = (size_t)g.npix_in * g.xw * 4;
     const size_t bit_bytes = (size_t)g.ocb * kh * kw * g.xw * g.q * 4;
-    g.use_mfma = mfma_applicable(g) ? 1 : 0;
+    g.cus = 256;
+    {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n,
+                    hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            g.cus = n;
+        else
+            (void)hipGetLastError();
+    }
+    g.mfma_ps = mfma_tile_blocks(g);
+    g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
     g.wfrag_offset = (bit_bytes + 255) / 256 * 256;
     c->resource_size[xnor_nn_resource_bin_weights] =
         g.use_mfma ? g.wfrag_offset + mfma_weight_bytes(g) : bit_bytes;

@@ -162,10 +162,7 @@ int pick_q(int oc, int xw) {
 
 const char *convolution_kernel_name(const Geometry &g) {
     static thread_local char name[64];
-    if (g.use_mfma) {
-        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d>", (g.ic + 63) / 64);
-        return name;
-    }
+    if (g.use_mfma) return mfma_kernel_name(g);
     const int xw = (g.xw == 3 || g.xw == 8 || g.xw == 12 || g.xw == 16) ? g.xw : 0;
     snprintf(name, sizeof name, "conv_xnor_popc_kernel<XW=%d,Q=%d>", xw, g.q);
     return name;

@@ -13,13 +13,20 @@
 // operand (columns): in the 32x32 accumulator layout a register then holds 32 consecutive
 // pixels of one filter, i.e. 128 contiguous bytes of the NCHW output.
 //
-// Workgroup = 128 consecutive output pixels x 128 filters, four waves of 64 x 64.
+// Workgroup = 32*PS consecutive output pixels x 256 filters; wave w owns filters
+// 64w .. 64w+63 for all pixels of the tile (2 x PS accumulator blocks of 32x32).
 //   * X: the packed sign bits of every input pixel the tile touches are expanded to FP4
 //     once and kept in LDS, one row per input pixel (channel-major, 16 spare bytes per row
-//     so that the 32 rows a fragment load touches spread over all banks).  A tap is a row
-//     offset; invalid taps point at a zero row.
+//     so that the rows a fragment load touches spread over all banks).  A tap is a row
+//     offset; invalid taps point at a zero row.  All four waves read the same rows.
 //   * W: pre-packed on the weight stage in fragment order (1 KB per 32 filters x 64
-//     channels), loaded straight into registers one tap ahead of use.
+//     channels), loaded straight into registers ahead of use.  A wave's two fragments
+//     per step feed 2*PS matrix instructions: with PS >= 3 the weight stream stays well
+//     below what the vector memory path of a compute unit delivers (with 2 x 2 blocking it
+//     ran at 80% of it and set the pace).
+//   * PS (2, 3 or 4) is chosen per problem so that the waves divide evenly over the SIMDs:
+//     for 43264 pixels, PS = 3 gives 1.76 waves per SIMD (2 in the busiest), PS = 4 gives
+//     1.32 (also 2, but each a third longer).
 #include <cstdlib>
 #include <type_traits>
 
@@ -33,19 +40,19 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int MT = 128;       // output pixels per workgroup
-constexpr int NT = 128;       // filters per workgroup
+constexpr int NT = 256;       // filters per workgroup (4 waves x 64)
 constexpr int ROW_PAD = 16;   // spare bytes per LDS row
 constexpr int TABLE_BYTES = 1024;
 constexpr int ALPHA_BYTES = NT * 4;
 constexpr int LDS_LIMIT = 64 * 1024;
 
-// First and last input pixel (flattened index) that the tile of MT output pixels starting
-// at tile*MT can touch with an in-bounds tap, for stride 1: from the start of the first
+// First and last input pixel (flattened index) that the tile of mt output pixels starting
+// at tile*mt can touch with an in-bounds tap, for stride 1: from the start of the first
 // input row of its first pixel to the end of the last input row of its last pixel.
-__host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, int &lo, int &hi) {
-    const uint32_t p_first = tile * MT;
-    uint32_t p_last = p_first + MT;
+__host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, uint32_t mt,
+        int &lo, int &hi) {
+    const uint32_t p_first = tile * mt;
+    uint32_t p_last = p_first + mt;
     if (p_last > g.npix_out) p_last = g.npix_out;
     p_last -= 1;
     const uint32_t i0 = p_first / g.ohw, i1 = p_last / g.ohw;
@@ -70,21 +77,31 @@ __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c)
 }
 
 // Weight fragments are fetched with hand-issued loads and hand-placed waits: left to
-// itself the compiler hoists the loads of the next tap to the top of the current one and
-// then waits for them before the first matrix instruction.
+// itself the compiler hoists the loads of the next group to the top of the current one
+// and then waits for them before the first matrix instruction.
 //   * load_frag_async only starts the load; the register holds the data once a later
 //     wait_loads_after() has run.
-//   * wait_loads_after() is "s_waitcnt vmcnt(0)" carrying the four accumulator tiles as
-//     read-write operands.  That data dependence orders it behind the matrix instructions
-//     issued before it and ahead of those that follow, which are the ones that consume
-//     the awaited fragments.  The fragments themselves are deliberately not operands: a
+//   * wait_loads_after() is "s_waitcnt vmcnt(0)" carrying accumulator blocks as read-write
+//     operands.  That data dependence orders it behind the matrix instructions issued
+//     before it and ahead of those that follow, which are the ones that consume the
+//     awaited fragments.  The fragments themselves are deliberately not operands: a
 //     read-write operand lets the compiler copy the register on the way in, and a copy of
 //     a register whose load is still in flight copies stale data.
 __device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src));
 }
-__device__ __forceinline__ void wait_loads_after(v16f &a, v16f &b, v16f &c, v16f &d) {
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+template <int PS>
+__device__ __forceinline__ void wait_loads_after(v16f (&acc)[2][PS]) {
+    if constexpr (PS == 2)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]),
+                "+v"(acc[1][1]));
+    else if constexpr (PS == 3)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]),
+                "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]));
+    else
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]),
+                "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]),
+                "+v"(acc[1][3]));
 }
 
 // FP4 codes of eight channels from one byte of packed sign bits (bit 7 = first channel,
@@ -97,8 +114,9 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
     return out;
 }
 
-// KS = 64-channel steps per tap = ceil(IC / 64).
-template <int KS, bool RAW>
+// KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4), PS = 32-pixel
+// blocks per workgroup tile.
+template <int KS, int PS, bool RAW>
 __global__ __launch_bounds__(256, 2)
 void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
@@ -109,6 +127,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
     unsigned char *rows = smem + TABLE_BYTES + ALPHA_BYTES; // row 0 is zero, then the tile
     constexpr int ROW_BYTES = KS * 32 + ROW_PAD;
+    constexpr int MT = 32 * PS;
+    // fragments are fetched in groups of HS steps: half a tap where that is >= 2 steps
+    constexpr int HS = (KS % 2 == 0 && KS >= 4) ? KS / 2 : KS;
+    constexpr int GROUPS_PER_TAP = KS / HS;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -120,13 +142,13 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // ---- which input pixels does the tile touch (stride 1) ----------------------------
     const uint32_t p_first = tile * MT;
     int lo, hi;
-    tile_span(g, tile, lo, hi);
+    tile_span(g, tile, MT, lo, hi);
     const int nrows = min(hi - lo + 1, max_rows);
 
     // ---- LDS: lookup table, zero row, this workgroup's alphas, FP4 rows ----------------------
     table[tid] = fp4_of_byte(tid);
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
-    if (tid < NT) {
+    {
         const int oc = chunk * NT + tid;
         alpha_lds[tid] = oc < g.oc ? alpha[oc] : 0.f;
     }
@@ -161,15 +183,15 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         }
     }
 
-    // ---- this wave's 64 filters x 64 pixels -------------------------------------------------
-    const int oc_sub0 = chunk * (NT / 32) + (wave & 1) * 2; // first 32-filter block
-    const uint32_t p_wave = p_first + (wave >> 1) * 64;
-    bool live[2];
-    int in0[2], oh[2], ow[2]; // input index of tap (0,0) relative to lo; output coordinates
-    uint32_t pix[2], img[2], rem[2];
+    // ---- this wave: 64 filters x 32*PS pixels --------------------------------------------------
+    const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
+    const bool wave_has_filters = oc_sub0 * 32 < g.oc; // wave-uniform
+    bool live[PS];
+    int in0[PS], oh[PS], ow[PS]; // input index of tap (0,0) relative to lo; output coordinates
+    uint32_t pix[PS], img[PS], rem[PS];
 #pragma unroll
-    for (int ps = 0; ps < 2; ps++) {
-        pix[ps] = p_wave + ps * 32 + (lane & 31);
+    for (int ps = 0; ps < PS; ps++) {
+        pix[ps] = p_first + ps * 32 + (lane & 31);
         live[ps] = pix[ps] < g.npix_out;
         const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
         img[ps] = g.div_ohw.div(pc);
@@ -180,73 +202,96 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     }
     const int half_off = (lane >> 5) * 16;
 
-    v16f acc[2][2];
+    v16f acc[2][PS];
 #pragma unroll
     for (int os = 0; os < 2; os++)
 #pragma unroll
-        for (int ps = 0; ps < 2; ps++)
+        for (int ps = 0; ps < PS; ps++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[os][ps][i] = 0.f;
 
-    // Weight fragments: [32-filter block][tap][step][lane], two register sets used in turn.
-    // The fragments of tap t+1 are requested before tap t is multiplied and awaited after
-    // its 4*KS matrix instructions; every request is awaited before the loop edge, so no
-    // register with a load in flight is live across it.
+    // Weight fragments: [32-filter block][tap][step][lane], two register sets of HS steps
+    // used in turn.  Group n+1 is requested before group n is multiplied and awaited after
+    // its 2*PS*HS matrix instructions; every request is awaited before the loop edge, so
+    // no register with a load in flight is live across it.
     const v4i *wsrc[2];
 #pragma unroll
     for (int os = 0; os < 2; os++)
         wsrc[os] = wfrag + (size_t)(oc_sub0 + os) * taps * KS * 64 + lane;
-    auto request_tap = [&](int t, v4i (&w)[KS][2]) {
+    auto request = [&](int group, v4i (&w)[HS][2]) { // group = tap * GROUPS_PER_TAP + part
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++)
+        for (int hs = 0; hs < HS; hs++)
 #pragma unroll
             for (int os = 0; os < 2; os++)
-                load_frag_async(w[ks][os], wsrc[os] + ((size_t)t * KS + ks) * 64);
+                load_frag_async(w[hs][os], wsrc[os] + ((size_t)group * HS + hs) * 64);
     };
-    auto multiply_tap = [&](int t, const v4i (&w)[KS][2]) {
+    int addr[PS];
+    auto tap_rows = [&](int t) { // LDS byte address of each pixel's row for tap t
         const int kh = t / g.kw, kw = t - kh * g.kw;
-        int addr[2];
 #pragma unroll
-        for (int ps = 0; ps < 2; ps++) {
+        for (int ps = 0; ps < PS; ps++) {
             const int ih = oh[ps] - g.ph + kh, iw = ow[ps] - g.pw + kw;
             const int r = in0[ps] + kh * g.iw + kw;
             const bool ok = live[ps] && (unsigned)ih < (unsigned)g.ih
                 && (unsigned)iw < (unsigned)g.iw && (unsigned)r < (unsigned)nrows;
             addr[ps] = (ok ? (1 + r) * ROW_BYTES : 0) + half_off;
         }
+    };
+    auto multiply = [&](const int part, const v4i (&w)[HS][2]) { // steps part*HS .. +HS-1
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            v4i b[2];
+        for (int hs = 0; hs < HS; hs++) {
+            v4i b[PS];
 #pragma unroll
-            for (int ps = 0; ps < 2; ps++)
-                b[ps] = *reinterpret_cast<const v4i *>(rows + addr[ps] + ks * 32);
+            for (int ps = 0; ps < PS; ps++)
+                b[ps] = *reinterpret_cast<const v4i *>(rows + addr[ps] + (part * HS + hs) * 32);
 #pragma unroll
             for (int os = 0; os < 2; os++)
 #pragma unroll
-                for (int ps = 0; ps < 2; ps++)
-                    acc[os][ps] = mfma_fp4(w[ks][os], b[ps], acc[os][ps]);
+                for (int ps = 0; ps < PS; ps++)
+                    acc[os][ps] = mfma_fp4(w[hs][os], b[ps], acc[os][ps]);
         }
     };
 
-    v4i wa[KS][2], wb[KS][2];
-    request_tap(0, wa);
-    wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]);
+    v4i wa[HS][2], wb[HS][2];
+    if (wave_has_filters) {
+        request(0, wa);
+        wait_loads_after<PS>(acc);
+    }
     __syncthreads(); // FP4 rows are in place
-    for (int t = 0; t < taps; t += 2) {
-        const bool second = t + 1 < taps, third = t + 2 < taps;
-        if (second) request_tap(t + 1, wb);
-        multiply_tap(t, wa);
-        if (second) {
-            wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]); // wb has landed
-            if (third) request_tap(t + 2, wa);
-            multiply_tap(t + 1, wb);
-            if (third) wait_loads_after(acc[0][0], acc[0][1], acc[1][0], acc[1][1]); // wa
+    if (wave_has_filters) {
+        if constexpr (GROUPS_PER_TAP == 2) {
+            for (int t = 0; t < taps; t++) {
+                tap_rows(t);
+                request(2 * t + 1, wb);
+                multiply(0, wa);
+                wait_loads_after<PS>(acc); // wb has landed
+                if (t + 1 < taps) request(2 * t + 2, wa);
+                multiply(1, wb);
+                if (t + 1 < taps) wait_loads_after<PS>(acc); // wa has landed
+            }
+        } else {
+            for (int t = 0; t < taps; t += 2) {
+                const bool second = t + 1 < taps, third = t + 2 < taps;
+                tap_rows(t);
+                if (second) request(t + 1, wb);
+                multiply(0, wa);
+                if (second) {
+                    wait_loads_after<PS>(acc); // wb has landed
+                    tap_rows(t + 1);
+                    if (third) request(t + 2, wa);
+                    multiply(0, wb);
+                    if (third) wait_loads_after<PS>(acc); // wa has landed
+                }
+            }
         }
     }
 
+    // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
+    //      pixel lane%32 ------------------------------------------------------------------------
+    if (!wave_has_filters) return;
     auto store_tile = [&](auto check_filters) {
 #pragma unroll
-        for (int ps = 0; ps < 2; ps++) {
+        for (int ps = 0; ps < PS; ps++) {
             if (!live[ps]) continue;
             const int n = opc[rem[ps]];
             const float kv = RAW ? 0.f : kplane[pix[ps]];
@@ -255,8 +300,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             for (int os = 0; os < 2; os++) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int ocl = ((wave & 1) * 2 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4
-                        + (i & 3);
+                    const int ocl = (wave * 2 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4 + (i & 3);
                     const int oc = chunk * NT + ocl;
                     if (decltype(check_filters)::value && oc >= g.oc) continue;
                     const float d = acc[os][ps][i]; // = 2*popc - n, exactly
@@ -274,7 +318,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             }
         }
     };
-    if ((chunk + 1) * NT <= g.oc) // workgroup-uniform: every filter of the chunk exists
+    if (chunk * NT + (wave + 1) * 64 <= g.oc) // wave-uniform: all 64 filters exist
         store_tile(std::false_type{});
     else
         store_tile(std::true_type{});
@@ -312,48 +356,89 @@ void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__
     frag[i] = out;
 }
 
-int steps_per_tap(const Geometry &g) { return (g.ic + 63) / 64; }
+// Steps per tap as the kernel is instantiated: ceil(IC/64), odd counts above 4 rounded up
+// (the extra step multiplies FP4 zeros).
+int steps_per_tap(const Geometry &g) {
+    const int ks = (g.ic + 63) / 64;
+    return ks > 4 && (ks & 1) ? ks + 1 : ks;
+}
 int oc_subblocks(const Geometry &g) { return ((g.oc + NT - 1) / NT) * (NT / 32); }
 
-// Largest number of input pixels any tile touches.  The offset of a tile within its image
-// repeats after at most OHW tiles, so that many (plus the last, possibly short, tile) are
-// enough to look at.
-int max_tile_rows(const Geometry &g) {
-    const uint32_t tiles = (g.npix_out + MT - 1) / MT;
+// Largest number of input pixels any tile of mt output pixels touches.  The offset of a
+// tile within its image repeats after at most OHW tiles, so that many (plus the last,
+// possibly short, tile) are enough to look at.
+int max_tile_rows(const Geometry &g, uint32_t mt) {
+    const uint32_t tiles = (g.npix_out + mt - 1) / mt;
     const uint32_t look = tiles < (uint32_t)g.ohw + 1 ? tiles : (uint32_t)g.ohw + 1;
     int most = 1;
     for (uint32_t t = 0; t < look; t++) {
         int lo, hi;
-        tile_span(g, t, lo, hi);
+        tile_span(g, t, mt, lo, hi);
         if (hi - lo + 1 > most) most = hi - lo + 1;
     }
     int lo, hi;
-    tile_span(g, tiles - 1, lo, hi);
+    tile_span(g, tiles - 1, mt, lo, hi);
     if (hi - lo + 1 > most) most = hi - lo + 1;
     return most;
 }
 
-size_t lds_bytes(const Geometry &g) {
-    return TABLE_BYTES + ALPHA_BYTES + (size_t)(1 + max_tile_rows(g)) * (steps_per_tap(g) * 32 + ROW_PAD);
+size_t lds_bytes(const Geometry &g, int ps) {
+    return TABLE_BYTES + ALPHA_BYTES
+        + (size_t)(1 + max_tile_rows(g, 32 * ps)) * (steps_per_tap(g) * 32 + ROW_PAD);
 }
 
-template <int KS>
+// 32-pixel blocks per tile: the choice that minimises (waves on the busiest SIMD) x (work
+// per wave); ties go to the larger tile, which streams fewer weight bytes.
+int pick_ps(const Geometry &g) {
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
+        const int v = atoi(e);
+        if (v >= 2 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT) return v;
+    }
+    const int chunks = (g.oc + NT - 1) / NT;
+    const int waves_per_block = g.oc >= NT ? 4 : (g.oc + 63) / 64;
+    const double simds = (double)g.cus * 4;
+    int best = 0;
+    double best_cost = 0;
+    for (int ps = 4; ps >= 2; ps--) {
+        if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
+        const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
+        const double per_simd = tiles * chunks * waves_per_block / simds;
+        const double busiest = per_simd <= 1 ? 1 : (double)(long)(per_simd + 0.999999);
+        const double cost = busiest * ps;
+        if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
+    }
+    return best;
+}
+
+template <int KS, int PS>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
         hipStream_t s) {
     const int chunks = (g.oc + NT - 1) / NT;
-    const uint32_t tiles = (g.npix_out + MT - 1) / MT;
+    const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
     const dim3 grid(tiles * chunks), block(256);
-    const int rows = max_tile_rows(g);
-    const size_t lds = lds_bytes(g);
+    const int rows = max_tile_rows(g, 32 * PS);
+    const size_t lds = lds_bytes(g, PS);
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (popc)
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, true>), grid, block, lds, s, xbits, wf,
-                alpha, k, opc, dst, popc, g, rows, chunks);
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true>), grid, block, lds, s, xbits,
+                wf, alpha, k, opc, dst, popc, g, rows, chunks);
     else
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, false>), grid, block, lds, s, xbits, wf,
-                alpha, k, opc, dst, popc, g, rows, chunks);
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false>), grid, block, lds, s, xbits,
+                wf, alpha, k, opc, dst, popc, g, rows, chunks);
     return hipGetLastError();
+}
+
+template <int KS>
+hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
+        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        hipStream_t s) {
+    switch (g.mfma_ps) {
+    case 2: return launch_mfma<KS, 2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 3: return launch_mfma<KS, 3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 4: return launch_mfma<KS, 4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    }
+    return hipErrorInvalidValue;
 }
 
 } // namespace
@@ -361,13 +446,14 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
 // The matrix-core kernel covers stride-1 convolutions with up to 512 input channels whose
 // tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
-bool mfma_applicable(const Geometry &g) {
+// Returns the tile size (32-pixel blocks per workgroup, 2..4) or 0 when not applicable.
+int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
-        if (e[0] == 'v') return false;
-    if (g.sh != 1 || g.sw != 1) return false;
-    if (steps_per_tap(g) > 8) return false;
-    if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return false;
-    return lds_bytes(g) <= (size_t)LDS_LIMIT;
+        if (e[0] == 'v') return 0;
+    if (g.sh != 1 || g.sw != 1) return 0;
+    if ((g.ic + 63) / 64 > 8) return 0;
+    if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
+    return pick_ps(g);
 }
 
 size_t mfma_weight_bytes(const Geometry &g) {
@@ -382,18 +468,22 @@ hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *
     return hipGetLastError();
 }
 
+const char *mfma_kernel_name(const Geometry &g) {
+    static thread_local char name[64];
+    snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d>", steps_per_tap(g), g.mfma_ps);
+    return name;
+}
+
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
         float *dst, int32_t *popc, hipStream_t s) {
     switch (steps_per_tap(g)) {
-    case 1: return launch_mfma<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 2: return launch_mfma<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 3: return launch_mfma<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 4: return launch_mfma<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 5: return launch_mfma<5>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 6: return launch_mfma<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 7: return launch_mfma<7>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 8: return launch_mfma<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
     }
     return hipErrorInvalidValue;
 }

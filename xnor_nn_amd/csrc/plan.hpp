@@ -52,7 +52,9 @@ struct Geometry {
     int ocb;      // ceil(oc/q)
     int ihw, ohw; // ih*iw, oh*ow
     uint32_t npix_in, npix_out; // mb*ihw, mb*ohw
+    int cus;                    // compute units of the device (256 if it cannot be asked)
     int use_mfma;               // 1: stage 3 runs the FP4 matrix-core kernel
+    int mfma_ps;                // its tile size in 32-pixel blocks (2..4)
     size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
@@ -86,7 +88,8 @@ hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         float *dst, int32_t *popc_or_null, hipStream_t s);
 hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
         hipStream_t s);
-bool mfma_applicable(const Geometry &g);
+int mfma_tile_blocks(const Geometry &g);
+const char *mfma_kernel_name(const Geometry &g);
 size_t mfma_weight_bytes(const Geometry &g);
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
         hipStream_t s);
