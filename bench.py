@@ -18,6 +18,11 @@ sys.path.insert(0, ROOT)
 
 METRIC = "ms/forward + effective binary GOPS, AlexNet conv4 N=256 on 1 MI355X"
 HBM_PEAK_GBS = 8000.0
+MFMA_FP4_PEAK_TOPS = 10100.0
+# HBM bytes per launch read from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch),
+# each scaled by what the same counter shows for a plain copy of known size; the runs and
+# the scale factors are recorded in profiles/.  Not measurable from inside this script.
+MEASURED_TRAFFIC = {}
 
 
 def work_figures(d):
@@ -40,6 +45,9 @@ def work_figures(d):
         "exact_ops": 2 * mb * oc * ic * taps,
         # fused binarize + mean|x| pass: read x once, write bits and a
         "binarize_bytes": 4 * mb * ic * ih * iw + mb * ih * iw * bic + 4 * mb * ih * iw,
+        # convolution: read packed input and FP4/packed weights once, k, write fp32 output
+        "conv_bytes": mb * ih * iw * bic + oc * kh * kw * bic + 4 * mb * oh * ow
+                      + 4 * mb * oc * oh * ow,
         # box filter: read a, write k
         "k_bytes": 4 * mb * ih * iw + 4 * mb * oh * ow,
         # whole stage 1+2 as the reference defines it when fused
@@ -162,9 +170,14 @@ def main():
     stage_ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i in range(3)]
     gpu_ms = sum(e[0].elapsed_time(e[3]) for e in evs) / args.steps
     conv_s = stage_ms[2] * 1e-3
-    # int32 VALU roofline of the convolution: one v_xnor_b32 + one v_bcnt_u32_b32 per lane
-    # handle 32 binary multiply-accumulates = 64 binary ops, so the chip's ceiling is
-    # CUs * 64 lanes * clock * 32 ops per lane-instruction.
+    # Roofline of the convolution kernel.  The matrix-core kernel multiplies +-1 values as
+    # FP4 operands, so its ceiling is the chip's dense FP4 MFMA rate.  The XNOR/popcount
+    # kernel (stride > 1, very wide inputs, or XNOR_NN_HIP_CONV=valu) is bounded by the
+    # integer VALU: one v_xnor_b32 + one v_bcnt_u32_b32 per lane handle 32 binary
+    # multiply-accumulates = 64 binary ops, i.e. CUs * 64 lanes * clock * 32 ops per
+    # lane-instruction.
+    conv_kernel = conv.kernel_name(0)
+    on_mfma = conv_kernel.startswith("conv_mfma")
     valu_peak_tops = cus * 64 * clk_hz * 32 / 1e12
     conv_tops = wf["exact_ops"] / conv_s / 1e12
     bin_gbs = wf["binarize_bytes"] / (stage_ms[0] * 1e-3) / 1e9
@@ -188,18 +201,29 @@ def main():
                      "forward": stage_ms[2]},
         "conv_effective_gops": wf["nominal_ops"] / conv_s / 1e9,
         "roofline": {
-            "kernel": conv.kernel_name(0), "bound": "valu",
-            "achieved": conv_tops, "peak": valu_peak_tops, "unit": "TOP/s",
-            "frac": conv_tops / valu_peak_tops, "traffic": None,
-            "peak_definition": "%d CUs x 64 lanes x %.3f GHz x 32 binary ops per VALU "
-                               "lane-instruction (xnor + bcnt pair = 64 ops)" % (
-                                   cus, clk_hz / 1e9),
+            "kernel": conv_kernel, "bound": "mfma" if on_mfma else "valu",
+            "achieved": conv_tops,
+            "peak": MFMA_FP4_PEAK_TOPS if on_mfma else valu_peak_tops,
+            "unit": "TFLOP/s",
+            "frac": conv_tops / (MFMA_FP4_PEAK_TOPS if on_mfma else valu_peak_tops),
+            "traffic": MEASURED_TRAFFIC.get((args.workload if args.mb is None else None,
+                                             conv_kernel.split("<")[0])),
+            "peak_definition": (
+                "MI355X dense FP4 MFMA rate, 10.1 PFLOP/s (signs are multiplied as FP4 +-1)"
+                if on_mfma else
+                "%d CUs x 64 lanes x %.3f GHz x 32 binary ops per VALU lane-instruction "
+                "(xnor + bcnt pair = 64 ops)" % (cus, clk_hz / 1e9)),
             "ops": "exact in-bounds binary ops per launch = %d" % wf["exact_ops"],
+            "hbm_view": {"bytes": wf["conv_bytes"],
+                         "achieved_gbs": wf["conv_bytes"] / conv_s / 1e9,
+                         "frac": wf["conv_bytes"] / conv_s / 1e9 / HBM_PEAK_GBS},
         },
         "roofline_binarize": {
             "kernel": conv.kernel_name(2), "bound": "hbm", "achieved": bin_gbs,
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bin_gbs / HBM_PEAK_GBS,
-            "bytes": wf["binarize_bytes"], "traffic": None,
+            "bytes": wf["binarize_bytes"],
+            "traffic": MEASURED_TRAFFIC.get((args.workload if args.mb is None else None,
+                                             conv.kernel_name(2).split("<")[0])),
             "stage1_plus_stage2": {"achieved": fused_gbs, "frac": fused_gbs / HBM_PEAK_GBS,
                                    "bytes": wf["fused_bytes"]},
         },
