@@ -121,7 +121,8 @@ __global__ __launch_bounds__(256, 2)
 void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
         const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
-        const Geometry g, const int max_rows, const int oc_chunks) {
+        const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
+        const uint32_t units_per_xcd) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
@@ -135,8 +136,13 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t tile = blockIdx.x / oc_chunks;
-    const int chunk = blockIdx.x - tile * oc_chunks;
+    // Workgroups are dealt to the eight XCDs round-robin: unit (b % 8) * units_per_xcd + b / 8
+    // gives each XCD one contiguous range of tiles, so the input rows two neighbouring tiles
+    // share and the output cache lines they both write into meet in one L2.
+    const uint32_t unit = (blockIdx.x & 7) * units_per_xcd + (blockIdx.x >> 3);
+    if (unit >= units) return;
+    const uint32_t tile = unit / oc_chunks;
+    const int chunk = unit - tile * oc_chunks;
     const int taps = g.kh * g.kw;
 
     // ---- which input pixels does the tile touch (stride 1) ----------------------------
@@ -287,33 +293,75 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     }
 
     // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
-    //      pixel lane%32 ------------------------------------------------------------------------
+    //      pixel lane%32.  Values are scaled in that layout; then v_permlane32_swap joins two
+    //      pixel blocks, so that a register holds 64 consecutive pixels of ONE filter and a
+    //      store instruction writes one 256-byte run of the NCHW output (the odd block of
+    //      PS = 3 keeps the 2 x 128-byte form).  The runs of one filter are stored back to
+    //      back so that the cache lines they share fill up in L2 before they can leave it. ----
     if (!wave_has_filters) return;
+    const int lane_hi = lane >> 5;
     auto store_tile = [&](auto check_filters) {
+        constexpr bool CHECK = decltype(check_filters)::value;
+        int n[PS];
+        float kv[PS];
+        size_t nchw0[PS];
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
-            if (!live[ps]) continue;
-            const int n = opc[rem[ps]];
-            const float kv = RAW ? 0.f : kplane[pix[ps]];
-            const size_t nchw0 = ((size_t)img[ps] * g.oc) * g.ohw + rem[ps];
+            n[ps] = opc[rem[ps]];
+            kv[ps] = RAW ? 0.f : kplane[live[ps] ? pix[ps] : 0];
+            nchw0[ps] = ((size_t)img[ps] * g.oc) * g.ohw + rem[ps];
+        }
+        // 64-pixel addressing of the joined blocks: pair q covers pixels 64q + lane
+        bool live64[PS / 2 > 0 ? PS / 2 : 1];
+        size_t at64[PS / 2 > 0 ? PS / 2 : 1];
 #pragma unroll
-            for (int os = 0; os < 2; os++) {
+        for (int q = 0; q < PS / 2; q++) {
+            const uint32_t p64 = p_first + q * 64 + lane;
+            live64[q] = p64 < g.npix_out;
+            const uint32_t pc = live64[q] ? p64 : g.npix_out - 1;
+            const uint32_t im = g.div_ohw.div(pc);
+            at64[q] = ((size_t)im * g.oc) * g.ohw + (pc - im * g.ohw);
+        }
+        const bool joined = RAW || g.dst_fmt == xnor_nn_data_format_nchw;
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int ocl = (wave * 2 + os) * 32 + 8 * (i / 4) + (lane >> 5) * 4 + (i & 3);
-                    const int oc = chunk * NT + ocl;
-                    if (decltype(check_filters)::value && oc >= g.oc) continue;
+        for (int os = 0; os < 2; os++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int oc_lo = (wave * 2 + os) * 32 + 8 * (i / 4) + (i & 3); // lanes 0..31
+                const int ocl = oc_lo + lane_hi * 4;
+                const int oc = chunk * NT + ocl;
+                uint32_t v[PS]; // bit patterns of the results in the accumulator layout
+#pragma unroll
+                for (int ps = 0; ps < PS; ps++) {
                     const float d = acc[os][ps][i]; // = 2*popc - n, exactly
-                    if constexpr (RAW) {
-                        popc[nchw0 + (size_t)oc * g.ohw] = ((int)d + n) / 2;
-                    } else {
-                        // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
-                        const float v = __fmul_rn(__fmul_rn(d, alpha_lds[ocl]), kv);
-                        if (g.dst_fmt == xnor_nn_data_format_nchw)
-                            dst[nchw0 + (size_t)oc * g.ohw] = v;
-                        else
-                            dst[(size_t)pix[ps] * g.oc + oc] = v;
+                    if constexpr (RAW)
+                        v[ps] = (uint32_t)(((int)d + n[ps]) / 2);
+                    else // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
+                        v[ps] = __float_as_uint(__fmul_rn(__fmul_rn(d, alpha_lds[ocl]), kv[ps]));
+                }
+                uint32_t *out = RAW ? reinterpret_cast<uint32_t *>(popc)
+                                    : reinterpret_cast<uint32_t *>(dst);
+                if (joined) {
+#pragma unroll
+                    for (int q = 0; q < PS / 2; q++) {
+                        const auto r = __builtin_amdgcn_permlane32_swap(v[2 * q], v[2 * q + 1],
+                                false, false);
+                        // r[0]: filter oc_lo, pixels 64q + lane; r[1]: filter oc_lo + 4
+                        const int oc_a = chunk * NT + oc_lo, oc_b = oc_a + 4;
+                        if (live64[q] && !(CHECK && oc_a >= g.oc))
+                            out[at64[q] + (size_t)oc_a * g.ohw] = r[0];
+                        if (live64[q] && !(CHECK && oc_b >= g.oc))
+                            out[at64[q] + (size_t)oc_b * g.ohw] = r[1];
                     }
+                    if constexpr (PS % 2 == 1) {
+                        if (live[PS - 1] && !(CHECK && oc >= g.oc))
+                            out[nchw0[PS - 1] + (size_t)oc * g.ohw] = v[PS - 1];
+                    }
+                } else {
+#pragma unroll
+                    for (int ps = 0; ps < PS; ps++)
+                        if (live[ps] && !(CHECK && oc >= g.oc))
+                            out[(size_t)pix[ps] * g.oc + oc] = v[ps];
                 }
             }
         }
@@ -416,16 +464,17 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         hipStream_t s) {
     const int chunks = (g.oc + NT - 1) / NT;
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
-    const dim3 grid(tiles * chunks), block(256);
+    const uint32_t units = tiles * chunks, per_xcd = (units + 7) / 8;
+    const dim3 grid(per_xcd * 8), block(256);
     const int rows = max_tile_rows(g, 32 * PS);
     const size_t lds = lds_bytes(g, PS);
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks);
+                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd);
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks);
+                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd);
     return hipGetLastError();
 }
 
