@@ -76,33 +76,60 @@ __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c)
             0x7f7f7f7f);
 }
 
-// Weight fragments are fetched with hand-issued loads and hand-placed waits: left to
-// itself the compiler hoists the loads of the next group to the top of the current one
-// and then waits for them before the first matrix instruction.
-//   * load_frag_async only starts the load; the register holds the data once a later
-//     wait_loads_after() has run.
-//   * wait_loads_after() is "s_waitcnt vmcnt(0)" carrying accumulator blocks as read-write
+// Operand traffic is issued by hand.  Left to itself the compiler hoists the global loads of
+// the next weight fragments to the top of the current group and then waits for them before
+// the first matrix instruction, and it sinks every LDS read to just ahead of its first use,
+// where the matrix pipe then idles for the whole LDS latency.
+//   * load_frag_async / fetch_rows_after only start loads; the destination registers hold
+//     data once a later wait has run.
+//   * Every wait is an "s_waitcnt" that carries the accumulator blocks as read-write
 //     operands.  That data dependence orders it behind the matrix instructions issued
 //     before it and ahead of those that follow, which are the ones that consume the
-//     awaited fragments.  The fragments themselves are deliberately not operands: a
-//     read-write operand lets the compiler copy the register on the way in, and a copy of
-//     a register whose load is still in flight copies stale data.
+//     awaited registers.  The awaited registers themselves are deliberately not operands
+//     of the wait: a read-write operand lets the compiler copy the register on the way in,
+//     and a copy of a register whose load is still in flight copies stale data.  For the
+//     same reason nothing is in flight when control passes a loop edge.
+//   * fetch_rows_after first waits for the LDS reads of the previous call (the operands of
+//     the matrix instructions that follow it) and then starts the reads for the step after,
+//     which the 2*PS matrix instructions of the current step cover.
 __device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src));
 }
+#define XNOR_ACC2 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1])
+#define XNOR_ACC3 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[1][0]), \
+        "+v"(acc[1][1]), "+v"(acc[1][2])
+#define XNOR_ACC4 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), \
+        "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3])
 template <int PS>
-__device__ __forceinline__ void wait_loads_after(v16f (&acc)[2][PS]) {
-    if constexpr (PS == 2)
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]),
-                "+v"(acc[1][1]));
-    else if constexpr (PS == 3)
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]),
-                "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]));
-    else
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]),
-                "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]),
-                "+v"(acc[1][3]));
+__device__ __forceinline__ void wait_all_after(v16f (&acc)[2][PS]) {
+    if constexpr (PS == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC2);
+    else if constexpr (PS == 3) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC3);
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC4);
 }
+template <int PS>
+__device__ __forceinline__ void fetch_rows_after(v4i (&bn)[PS], const uint32_t (&a)[PS],
+        v16f (&acc)[2][PS]) {
+    if constexpr (PS == 2)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+                     "ds_read_b128 %[b1], %[a1]"
+                : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), XNOR_ACC2
+                : [a0] "v"(a[0]), [a1] "v"(a[1]));
+    else if constexpr (PS == 3)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+                     "ds_read_b128 %[b1], %[a1]\n\tds_read_b128 %[b2], %[a2]"
+                : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), [b2] "=&v"(bn[2]), XNOR_ACC3
+                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+                     "ds_read_b128 %[b1], %[a1]\n\tds_read_b128 %[b2], %[a2]\n\t"
+                     "ds_read_b128 %[b3], %[a3]"
+                : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), [b2] "=&v"(bn[2]), [b3] "=&v"(bn[3]),
+                  XNOR_ACC4
+                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]));
+}
+#undef XNOR_ACC2
+#undef XNOR_ACC3
+#undef XNOR_ACC4
 
 // FP4 codes of eight channels from one byte of packed sign bits (bit 7 = first channel,
 // set = sign bit clear = +1): nibble i = channel i, +1 -> 0x2, -1 -> 0xA.
@@ -217,9 +244,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             for (int i = 0; i < 16; i++) acc[os][ps][i] = 0.f;
 
     // Weight fragments: [32-filter block][tap][step][lane], two register sets of HS steps
-    // used in turn.  Group n+1 is requested before group n is multiplied and awaited after
-    // its 2*PS*HS matrix instructions; every request is awaited before the loop edge, so
-    // no register with a load in flight is live across it.
+    // used in turn (a "group" is HS steps of one tap).  Group n+1 is requested before group
+    // n is multiplied and awaited after its 2*PS*HS matrix instructions.
     const v4i *wsrc[2];
 #pragma unroll
     for (int os = 0; os < 2; os++)
@@ -231,65 +257,91 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             for (int os = 0; os < 2; os++)
                 load_frag_async(w[hs][os], wsrc[os] + ((size_t)group * HS + hs) * 64);
     };
-    int addr[PS];
-    auto tap_rows = [&](int t) { // LDS byte address of each pixel's row for tap t
+    const uint32_t rows_base = (uint32_t)(size_t)rows; // LDS byte offset of the zero row
+    auto tap_rows = [&](int t, uint32_t (&out)[PS]) { // LDS address of each pixel's row
         const int kh = t / g.kw, kw = t - kh * g.kw;
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
             const int ih = oh[ps] - g.ph + kh, iw = ow[ps] - g.pw + kw;
             const int r = in0[ps] + kh * g.iw + kw;
-            const bool ok = live[ps] && (unsigned)ih < (unsigned)g.ih
-                && (unsigned)iw < (unsigned)g.iw && (unsigned)r < (unsigned)nrows;
-            addr[ps] = (ok ? (1 + r) * ROW_BYTES : 0) + half_off;
+            const bool ok = (int)live[ps] & (int)((unsigned)ih < (unsigned)g.ih)
+                & (int)((unsigned)iw < (unsigned)g.iw) & (int)((unsigned)r < (unsigned)nrows);
+            out[ps] = rows_base + (ok ? (1 + r) * ROW_BYTES : 0) + half_off;
         }
     };
-    auto multiply = [&](const int part, const v4i (&w)[HS][2]) { // steps part*HS .. +HS-1
+    auto mma = [&](const v4i (&w)[2], const v4i (&b)[PS]) {
 #pragma unroll
-        for (int hs = 0; hs < HS; hs++) {
-            v4i b[PS];
+        for (int os = 0; os < 2; os++)
 #pragma unroll
             for (int ps = 0; ps < PS; ps++)
-                b[ps] = *reinterpret_cast<const v4i *>(rows + addr[ps] + (part * HS + hs) * 32);
+                acc[os][ps] = mfma_fp4(w[os], b[ps], acc[os][ps]);
+    };
+
+    const int last_group = taps * GROUPS_PER_TAP - 1;
+    uint32_t rowaddr[PS]; // rows of the current group's tap
+    v4i b0[PS], b1[PS];   // pixel fragments of the current and the following step, in turn
+    // One group with the fragments in wc, while those of the next group arrive in wn.
+    // P0: which of b0/b1 holds the group's first step; OFF / NOFF: byte offset within a row of
+    // this group's and of the next group's first step.  In the paired loop the group after
+    // the last one is the last one again: loaded, awaited and never used.  MORE = false (the
+    // single group after the loop) fetches nothing beyond the group: a load whose result is
+    // never read must not exist, because its destination registers would be given to
+    // something else while it is still in flight.
+    auto run_group = [&](auto more, auto p0, auto off, auto noff, int n,
+                         const v4i (&wc)[HS][2], v4i (&wn)[HS][2]) {
+        constexpr bool MORE = decltype(more)::value;
+        constexpr int P0 = decltype(p0)::value, OFF = decltype(off)::value,
+                      NOFF = decltype(noff)::value;
+        uint32_t nextaddr[PS];
+        if constexpr (MORE) {
+            const int next = min(n + 1, last_group);
+            request(next, wn);
+            tap_rows(next / GROUPS_PER_TAP, nextaddr);
+        }
 #pragma unroll
-            for (int os = 0; os < 2; os++)
+        for (int hs = 0; hs < HS; hs++) {
+            if (hs + 1 < HS || MORE) {
+                uint32_t a[PS];
 #pragma unroll
                 for (int ps = 0; ps < PS; ps++)
-                    acc[os][ps] = mfma_fp4(w[hs][os], b[ps], acc[os][ps]);
+                    a[ps] = hs + 1 < HS ? rowaddr[ps] + OFF + (hs + 1) * 32
+                                        : nextaddr[ps] + NOFF;
+                if (((P0 + hs) & 1) == 0) fetch_rows_after<PS>(b1, a, acc);
+                else fetch_rows_after<PS>(b0, a, acc);
+            } else {
+                wait_all_after<PS>(acc); // the last fragments of the kernel are in
+            }
+            if (((P0 + hs) & 1) == 0) mma(wc[hs], b0);
+            else mma(wc[hs], b1);
+        }
+        if constexpr (MORE) {
+            wait_all_after<PS>(acc); // wn and the first pixel fragments of the next group are in
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) rowaddr[ps] = nextaddr[ps];
         }
     };
 
     v4i wa[HS][2], wb[HS][2];
     if (wave_has_filters) {
         request(0, wa);
-        wait_loads_after<PS>(acc);
+        tap_rows(0, rowaddr);
     }
     __syncthreads(); // FP4 rows are in place
     if (wave_has_filters) {
-        if constexpr (GROUPS_PER_TAP == 2) {
-            for (int t = 0; t < taps; t++) {
-                tap_rows(t);
-                request(2 * t + 1, wb);
-                multiply(0, wa);
-                wait_loads_after<PS>(acc); // wb has landed
-                if (t + 1 < taps) request(2 * t + 2, wa);
-                multiply(1, wb);
-                if (t + 1 < taps) wait_loads_after<PS>(acc); // wa has landed
-            }
-        } else {
-            for (int t = 0; t < taps; t += 2) {
-                const bool second = t + 1 < taps, third = t + 2 < taps;
-                tap_rows(t);
-                if (second) request(t + 1, wb);
-                multiply(0, wa);
-                if (second) {
-                    wait_loads_after<PS>(acc); // wb has landed
-                    tap_rows(t + 1);
-                    if (third) request(t + 2, wa);
-                    multiply(0, wb);
-                    if (third) wait_loads_after<PS>(acc); // wa has landed
-                }
-            }
+        fetch_rows_after<PS>(b0, rowaddr, acc);
+        wait_all_after<PS>(acc);
+        constexpr int P1 = HS & 1, OFF1 = GROUPS_PER_TAP == 2 ? HS * 32 : 0;
+        using std::integral_constant;
+        int n = 0;
+        for (; n + 1 <= last_group; n += 2) {
+            run_group(std::true_type{}, integral_constant<int, 0>{},
+                    integral_constant<int, 0>{}, integral_constant<int, OFF1>{}, n, wa, wb);
+            run_group(std::true_type{}, integral_constant<int, P1>{},
+                    integral_constant<int, OFF1>{}, integral_constant<int, 0>{}, n + 1, wb, wa);
         }
+        if (n <= last_group) // odd number of groups (only with one group per tap)
+            run_group(std::false_type{}, integral_constant<int, 0>{},
+                    integral_constant<int, 0>{}, integral_constant<int, 0>{}, n, wa, wb);
     }
 
     // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
