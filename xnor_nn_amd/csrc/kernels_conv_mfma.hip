@@ -220,7 +220,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
     const bool wave_has_filters = oc_sub0 * 32 < g.oc; // wave-uniform
     bool live[PS];
-    int in0[PS], oh[PS], ow[PS]; // input index of tap (0,0) relative to lo; output coordinates
+    // Per pixel: LDS address of the row of tap (0,0), and which kernel rows / columns fall
+    // inside the image (bit kh of rowmask, bit kw of colmask; no bits for a dead pixel).
+    uint32_t base_addr[PS], rowmask[PS], colmask[PS];
     uint32_t pix[PS], img[PS], rem[PS];
 #pragma unroll
     for (int ps = 0; ps < PS; ps++) {
@@ -229,11 +231,22 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
         img[ps] = g.div_ohw.div(pc);
         rem[ps] = pc - img[ps] * g.ohw;
-        oh[ps] = (int)g.div_ow.div(rem[ps]);
-        ow[ps] = (int)rem[ps] - oh[ps] * g.ow;
-        in0[ps] = (int)(img[ps] * g.ihw) + (oh[ps] - g.ph) * g.iw + (ow[ps] - g.pw) - lo;
+        const int oh = (int)g.div_ow.div(rem[ps]);
+        const int ow = (int)rem[ps] - oh * g.ow;
+        const int in0 = (int)(img[ps] * g.ihw) + (oh - g.ph) * g.iw + (ow - g.pw) - lo;
+        base_addr[ps] = (uint32_t)(size_t)rows + (uint32_t)((1 + in0) * ROW_BYTES)
+            + (lane >> 5) * 16;
+        // kernel rows kh with 0 <= oh - ph + kh < ih, as a run of bits (kh < 32)
+        auto run_of_bits = [](int first, int last) -> uint32_t { // bits first..last, clipped
+            if (first < 0) first = 0;
+            if (last > 31) last = 31;
+            if (last < first) return 0u;
+            return (uint32_t)(((1ull << (last + 1)) - 1) & ~((1ull << first) - 1));
+        };
+        rowmask[ps] = live[ps] ? run_of_bits(g.ph - oh, g.ih - 1 + g.ph - oh) : 0u;
+        colmask[ps] = run_of_bits(g.pw - ow, g.iw - 1 + g.pw - ow);
     }
-    const int half_off = (lane >> 5) * 16;
+    const uint32_t zero_addr = (uint32_t)(size_t)rows + (lane >> 5) * 16;
 
     v16f acc[2][PS];
 #pragma unroll
@@ -257,17 +270,21 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             for (int os = 0; os < 2; os++)
                 load_frag_async(w[hs][os], wsrc[os] + ((size_t)group * HS + hs) * 64);
     };
-    const uint32_t rows_base = (uint32_t)(size_t)rows; // LDS byte offset of the zero row
-    auto tap_rows = [&](int t, uint32_t (&out)[PS]) { // LDS address of each pixel's row
-        const int kh = t / g.kw, kw = t - kh * g.kw;
+    // LDS address of each pixel's row for tap (kh, kw): a fixed offset from the row of tap
+    // (0,0), or the zero row when the tap falls outside the image.  Every in-bounds tap of a
+    // tile lies inside the span of rows the tile has staged (tile_span).
+    auto tap_rows = [&](int kh, int kw, uint32_t (&out)[PS]) {
+        const uint32_t shift = (uint32_t)((kh * g.iw + kw) * ROW_BYTES);
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
-            const int ih = oh[ps] - g.ph + kh, iw = ow[ps] - g.pw + kw;
-            const int r = in0[ps] + kh * g.iw + kw;
-            const bool ok = (int)live[ps] & (int)((unsigned)ih < (unsigned)g.ih)
-                & (int)((unsigned)iw < (unsigned)g.iw) & (int)((unsigned)r < (unsigned)nrows);
-            out[ps] = rows_base + (ok ? (1 + r) * ROW_BYTES : 0) + half_off;
+            const uint32_t ok = (rowmask[ps] >> kh) & (colmask[ps] >> kw) & 1u;
+            out[ps] = ok ? base_addr[ps] + shift : zero_addr;
         }
+    };
+    int nkh = 0, nkw = 0; // the tap after the one being multiplied (the last tap repeats)
+    auto advance_tap = [&]() {
+        if (nkw + 1 < g.kw) nkw++;
+        else if (nkh + 1 < g.kh) { nkw = 0; nkh++; }
     };
     auto mma = [&](const v4i (&w)[2], const v4i (&b)[PS]) {
 #pragma unroll
@@ -287,16 +304,21 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // single group after the loop) fetches nothing beyond the group: a load whose result is
     // never read must not exist, because its destination registers would be given to
     // something else while it is still in flight.
-    auto run_group = [&](auto more, auto p0, auto off, auto noff, int n,
+    auto run_group = [&](auto more, auto newtap, auto p0, auto off, auto noff, int n,
                          const v4i (&wc)[HS][2], v4i (&wn)[HS][2]) {
-        constexpr bool MORE = decltype(more)::value;
+        constexpr bool MORE = decltype(more)::value, NEWTAP = decltype(newtap)::value;
         constexpr int P0 = decltype(p0)::value, OFF = decltype(off)::value,
                       NOFF = decltype(noff)::value;
         uint32_t nextaddr[PS];
         if constexpr (MORE) {
-            const int next = min(n + 1, last_group);
-            request(next, wn);
-            tap_rows(next / GROUPS_PER_TAP, nextaddr);
+            request(min(n + 1, last_group), wn);
+            if constexpr (NEWTAP) { // the next group starts the next tap
+                tap_rows(nkh, nkw, nextaddr);
+                advance_tap();
+            } else {
+#pragma unroll
+                for (int ps = 0; ps < PS; ps++) nextaddr[ps] = rowaddr[ps];
+            }
         }
 #pragma unroll
         for (int hs = 0; hs < HS; hs++) {
@@ -324,7 +346,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     v4i wa[HS][2], wb[HS][2];
     if (wave_has_filters) {
         request(0, wa);
-        tap_rows(0, rowaddr);
+        tap_rows(0, 0, rowaddr);
+        advance_tap();
     }
     __syncthreads(); // FP4 rows are in place
     if (wave_has_filters) {
@@ -334,13 +357,14 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         using std::integral_constant;
         int n = 0;
         for (; n + 1 <= last_group; n += 2) {
-            run_group(std::true_type{}, integral_constant<int, 0>{},
-                    integral_constant<int, 0>{}, integral_constant<int, OFF1>{}, n, wa, wb);
-            run_group(std::true_type{}, integral_constant<int, P1>{},
+            run_group(std::true_type{}, integral_constant<bool, GROUPS_PER_TAP == 1>{},
+                    integral_constant<int, 0>{}, integral_constant<int, 0>{},
+                    integral_constant<int, OFF1>{}, n, wa, wb);
+            run_group(std::true_type{}, std::true_type{}, integral_constant<int, P1>{},
                     integral_constant<int, OFF1>{}, integral_constant<int, 0>{}, n + 1, wb, wa);
         }
         if (n <= last_group) // odd number of groups (only with one group per tap)
-            run_group(std::false_type{}, integral_constant<int, 0>{},
+            run_group(std::false_type{}, std::false_type{}, integral_constant<int, 0>{},
                     integral_constant<int, 0>{}, integral_constant<int, 0>{}, n, wa, wb);
     }
 
@@ -553,6 +577,7 @@ int mfma_tile_blocks(const Geometry &g) {
         if (e[0] == 'v') return 0;
     if (g.sh != 1 || g.sw != 1) return 0;
     if ((g.ic + 63) / 64 > 8) return 0;
+    if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
     if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
     return pick_ps(g);
 }
