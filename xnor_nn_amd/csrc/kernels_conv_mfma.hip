@@ -149,7 +149,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const float *__restrict__ alpha, const float *__restrict__ kplane,
         const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
         const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
-        const uint32_t units_per_xcd) {
+        const uint32_t units_per_xcd, const FastDiv div_xw) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
@@ -179,6 +179,19 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const int nrows = min(hi - lo + 1, max_rows);
 
     // ---- LDS: lookup table, zero row, this workgroup's alphas, FP4 rows ----------------------
+    // The rows of the tile are contiguous in the packed input: item i is word i of that
+    // run.  The first EARLY loads of every thread are in flight while the table is built.
+    // Words past ceil(IC/32) of a row are left as they are: the matching weights are FP4
+    // zeros and FP4 has no NaN or infinity, so whatever LDS holds there contributes nothing.
+    const int nitems = nrows * g.xw;
+    const uint32_t *run = xbits + (size_t)lo * g.xw;
+    constexpr int EARLY = 8;
+    uint32_t early[EARLY];
+#pragma unroll
+    for (int u = 0; u < EARLY; u++) {
+        const int i = u * 256 + tid;
+        early[u] = i < nitems ? run[i] : 0u;
+    }
     table[tid] = fp4_of_byte(tid);
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
     {
@@ -186,33 +199,31 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         alpha_lds[tid] = oc < g.oc ? alpha[oc] : 0.f;
     }
     __syncthreads();
-    // The rows of the tile are contiguous in the packed input: item i is word i of that
-    // run.  Four loads per thread are issued before the first is expanded.  Words past
-    // ceil(IC/32) of a row are left as they are: the matching weights are FP4 zeros and
-    // FP4 has no NaN or infinity, so whatever LDS holds there contributes nothing.
-    {
-        const int nitems = nrows * g.xw;
-        const uint32_t *run = xbits + (size_t)lo * g.xw;
-        for (int base = 0; base < nitems; base += 4 * 256) {
-            uint32_t w[4];
+    auto expand = [&](int i, uint32_t word) { // item i of the run -> 32 FP4 codes of its row
+        const int r = (int)div_xw.div((uint32_t)i), j = i - r * g.xw; // row, 32-channel word
+        v4i q;
+        q.x = table[word >> 24];
+        q.y = table[(word >> 16) & 0xFF];
+        q.z = table[(word >> 8) & 0xFF];
+        q.w = table[word & 0xFF];
+        *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
+    };
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int i = base + u * 256 + tid;
-                w[u] = i < nitems ? run[i] : 0u;
-            }
+    for (int u = 0; u < EARLY; u++) {
+        const int i = u * 256 + tid;
+        if (i < nitems) expand(i, early[u]);
+    }
+    for (int base = EARLY * 256; base < nitems; base += 4 * 256) {
+        uint32_t w[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int i = base + u * 256 + tid;
-                if (i < nitems) {
-                    const int r = i / g.xw, j = i - r * g.xw; // row, 32-channel word
-                    v4i q;
-                    q.x = table[w[u] >> 24];
-                    q.y = table[(w[u] >> 16) & 0xFF];
-                    q.z = table[(w[u] >> 8) & 0xFF];
-                    q.w = table[w[u] & 0xFF];
-                    *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
-                }
-            }
+        for (int u = 0; u < 4; u++) {
+            const int i = base + u * 256 + tid;
+            w[u] = i < nitems ? run[i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = base + u * 256 + tid;
+            if (i < nitems) expand(i, w[u]);
         }
     }
 
@@ -547,10 +558,12 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd);
+                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                FastDiv::make((uint32_t)g.xw));
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd);
+                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                FastDiv::make((uint32_t)g.xw));
     return hipGetLastError();
 }
 
