@@ -158,15 +158,23 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    # Timed region: exactly K steps, nothing but the three executor calls per step.
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(evs[i])
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-
     ms_per_step = 1e3 * (t1 - t0) / args.steps
+
+    # Second pass of K steps with HIP events around every stage, for the per-stage and
+    # roofline figures.  Each event record costs the stream a few microseconds, which is why
+    # this pass is not the one "value" is taken from.
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
     stage_ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i in range(3)]
     gpu_ms = sum(e[0].elapsed_time(e[3]) for e in evs) / args.steps
     conv_s = stage_ms[2] * 1e-3
@@ -196,7 +204,9 @@ def main():
                    "shape": {k: d[k] for k in ("mb", "ic", "ih", "iw", "oc", "kh", "kw",
                                                "sh", "sw", "ph", "pw")},
                    "layout": "NCHW/OIHW/NCHW", "weights_binarized": "once, outside the step"},
-        "gpu_ms_per_forward": gpu_ms,
+        "timing": "ms_per_step: wall clock over the K steps, no events inside; stage_ms and the "
+                  "rooflines: a second pass of K steps with HIP events around each stage",
+        "gpu_ms_per_forward_with_events": gpu_ms,
         "stage_ms": {"binarize_data": stage_ms[0], "calculate_k": stage_ms[1],
                      "forward": stage_ms[2]},
         "conv_effective_gops": wf["nominal_ops"] / conv_s / 1e9,

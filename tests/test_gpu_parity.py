@@ -219,6 +219,49 @@ def test_calculate_k_alone_matches_fused_path(oracle, gpu):
     conv.close()
 
 
+def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
+    """With the matrix-core kernel, calculate_k leaves the box filter to the convolution.
+    The K plane must still be what calculate_k saw: (1) read back before any forward, (2)
+    after the input and mean|x| were overwritten by a later binarize_data, (3) after a
+    forward, where the convolution kernel itself wrote it, and (4) with the deferral
+    switched off."""
+    import torch
+    d, x1, w = synth.make_workload("alexnet_conv4_mb256", 6)
+    x2 = (x1[::-1] * np.float32(1.5)).copy()
+    s = oracle_shape(oracle, d)
+    want1 = oracle.forward(s, x1, w)
+    want2 = oracle.forward(s, x2, w)
+    x1t, x2t = torch.from_numpy(x1).to(gpu), torch.from_numpy(x2).to(gpu)
+    dt = torch.empty(want1["dst"].shape, dtype=torch.float32, device=gpu)
+    conv = make(d, torch.from_numpy(w).to(gpu))
+    # (1)
+    conv.stage("binarize_data", src=x1t, dst=dt)
+    conv.stage("calculate_k")
+    assert np.array_equal(conv.export_floats(capi.RES_K), want1["k"])
+    # (2) K of x1 is owed when x2 is binarized; forward must then use K(x1) with bits(x2)
+    conv.stage("binarize_data", src=x1t)
+    conv.stage("calculate_k")
+    conv.stage("binarize_data", src=x2t)
+    assert np.array_equal(conv.export_floats(capi.RES_K), want1["k"])
+    assert np.array_equal(conv.export_floats(capi.RES_A), want2["a"])
+    # (3)
+    conv.stage("calculate_k")
+    conv.stage("forward")
+    conv.synchronize()
+    assert np.array_equal(dt.cpu().numpy().view(np.uint32), want2["dst"].view(np.uint32))
+    assert np.array_equal(conv.export_floats(capi.RES_K), want2["k"])
+    # (4)
+    monkeypatch.setenv("XNOR_NN_HIP_SEPARATE_K", "1")
+    dt.zero_()
+    conv.stage("binarize_data", src=x1t)
+    conv.stage("calculate_k")
+    conv.stage("forward")
+    conv.synchronize()
+    assert np.array_equal(dt.cpu().numpy().view(np.uint32), want1["dst"].view(np.uint32))
+    assert np.array_equal(conv.export_floats(capi.RES_K), want1["k"])
+    conv.close()
+
+
 def test_linearity_of_scaling_at_full_size(gpu):
     """Size-independent property at benchmark size: scaling the input by 2 leaves the
     packed bits and popcounts unchanged and doubles dst exactly (k is linear in |x| and

@@ -55,6 +55,18 @@ xnor_nn_status_t unimplemented_stage(const xnor_nn_convolution_t *, xnor_nn_reso
     return xnor_nn_unimplemented;
 }
 
+// Runs the box filter that calculate_k left to the convolution (see State::k_owed_a).
+xnor_nn_status_t settle_k(State *st) {
+    if (st->k_owed_a == nullptr) return xnor_nn_success;
+    const float *a = st->k_owed_a;
+    float *k = st->k_owed_k;
+    st->k_owed_a = nullptr;
+    st->k_owed_k = nullptr;
+    if (st->verbose) printf("xnor_nn exec (deferred calculate_k): box_filter_kernel\n");
+    return launch_box_filter(st->g, a, k, st->stream) == hipSuccess ? xnor_nn_success
+                                                                    : xnor_nn_error_memory;
+}
+
 // ---- stage 1 --------------------------------------------------------------------------
 // Replaces reference src/bcast_binarize_data.cpp:13-76 (same null checks, same
 // "unimplemented" for an unknown format).
@@ -69,6 +81,10 @@ xnor_nn_status_t exec_binarize_data(const xnor_nn_convolution_t *c, xnor_nn_reso
             src_elems(st->g) * sizeof(float), &x);
     if (rc != xnor_nn_success) return rc;
     float *a = static_cast<float *>(res[xnor_nn_resource_a]); // optional by-product
+    if (a != nullptr && a == st->k_owed_a) { // about to overwrite the mean|x| a K is owed from
+        rc = settle_k(st);
+        if (rc != xnor_nn_success) return rc;
+    }
     if (st->verbose) printf("xnor_nn exec binarize_data: %s\n", binarize_kernel_name(st->g));
     if (launch_binarize_data(st->g, static_cast<const float *>(x),
                 static_cast<uint32_t *>(res[xnor_nn_resource_bin_src]), a, st->stream)
@@ -93,6 +109,8 @@ xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resour
     const bool a_ready = st->a_ready_src == res[xnor_nn_resource_user_src]
         && st->a_ready_buf == a && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr;
     st->a_ready_src = st->a_ready_buf = nullptr; // one-shot
+    xnor_nn_status_t owed = settle_k(st); // an earlier, still deferred K (other buffers)
+    if (owed != xnor_nn_success) return owed;
     if (!a_ready) {
         const void *x = nullptr;
         xnor_nn_status_t rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
@@ -100,6 +118,16 @@ xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resour
         if (rc != xnor_nn_success) return rc;
         if (launch_mean_abs(st->g, static_cast<const float *>(x), a, st->stream) != hipSuccess)
             return xnor_nn_error_memory;
+    }
+    // The matrix-core convolution sums K from mean|x| itself, which saves this launch; the
+    // K plane is then written by the forward executor (or by whatever needs it earlier).
+    if (st->g.use_mfma && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr) {
+        if (st->verbose)
+            printf("xnor_nn exec calculate_k: %sbox filter deferred to the convolution\n",
+                    a_ready ? "" : "mean_abs, ");
+        st->k_owed_a = a;
+        st->k_owed_k = static_cast<float *>(res[xnor_nn_resource_k]);
+        return xnor_nn_success;
     }
     if (st->verbose)
         printf("xnor_nn exec calculate_k: %sbox_filter_kernel\n", a_ready ? "" : "mean_abs + ");
@@ -151,19 +179,40 @@ xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resourc
             return xnor_nn_error_memory;
         out = st->stage_dst;
     }
-    if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
-    const uint32_t *wbits = static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]);
-    if (st->g.use_mfma)
-        wbits = reinterpret_cast<const uint32_t *>(
+    const uint32_t *xbits = static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]);
+    const float *alpha = static_cast<const float *>(res[xnor_nn_resource_alpha]);
+    const float *k = static_cast<const float *>(res[xnor_nn_resource_k]);
+    const int32_t *opc = static_cast<const int32_t *>(res[xnor_nn_resource_operations_count]);
+    float *dst = raw ? nullptr : static_cast<float *>(out);
+    int32_t *popc = raw ? static_cast<int32_t *>(out) : nullptr;
+    hipError_t err;
+    if (st->g.use_mfma) {
+        const uint32_t *wfrag = reinterpret_cast<const uint32_t *>(
                 static_cast<const char *>(res[xnor_nn_resource_bin_weights]) + st->g.wfrag_offset);
-    if ((st->g.use_mfma ? launch_convolution_mfma : launch_convolution)(st->g,
-                static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]), wbits,
-                static_cast<const float *>(res[xnor_nn_resource_alpha]),
-                static_cast<const float *>(res[xnor_nn_resource_k]),
-                static_cast<const int32_t *>(res[xnor_nn_resource_operations_count]),
-                raw ? nullptr : static_cast<float *>(out),
-                raw ? static_cast<int32_t *>(out) : nullptr, st->stream) != hipSuccess)
-        return xnor_nn_error_memory;
+        // a K owed for exactly this K buffer is computed inside the kernel
+        const float *a = nullptr;
+        if (!raw && st->k_owed_a != nullptr) {
+            if (st->k_owed_k == k) {
+                a = st->k_owed_a;
+                st->k_owed_a = nullptr;
+                st->k_owed_k = nullptr;
+            } else {
+                xnor_nn_status_t rc = settle_k(st);
+                if (rc != xnor_nn_success) return rc;
+            }
+        }
+        if (st->verbose)
+            printf("xnor_nn exec forward: %s%s\n", convolution_kernel_name(st->g),
+                    a ? " (with the box filter of calculate_k)" : "");
+        err = launch_convolution_mfma(st->g, xbits, wfrag, alpha, k, opc, dst, popc, a,
+                const_cast<float *>(k), st->stream);
+    } else {
+        if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
+        err = launch_convolution(st->g, xbits,
+                static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]), alpha, k, opc,
+                dst, popc, st->stream);
+    }
+    if (err != hipSuccess) return xnor_nn_error_memory;
     if (!direct) {
         if (hipMemcpyAsync(user_out, out, bytes, hipMemcpyDeviceToHost, st->stream) != hipSuccess
                 || hipStreamSynchronize(st->stream) != hipSuccess)
@@ -436,6 +485,10 @@ xnor_nn_status_t xnor_nn_hip_export_floats(const xnor_nn_convolution_t *c,
             && slot != xnor_nn_resource_k)
         return xnor_nn_error_invalid_input;
     if (!res[slot] || dst_bytes != c->resource_size[slot]) return xnor_nn_error_invalid_input;
+    if (slot == xnor_nn_resource_k) { // a deferred box filter has to run before K is read
+        xnor_nn_status_t rc = settle_k(state_of(c));
+        if (rc != xnor_nn_success) return rc;
+    }
     return to_host(c, res[slot], dst, dst_bytes);
 }
 

@@ -149,12 +149,16 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const float *__restrict__ alpha, const float *__restrict__ kplane,
         const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
         const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
-        const uint32_t units_per_xcd, const FastDiv div_xw) {
+        const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
+        float *__restrict__ k_out, const float inv_khw) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
     unsigned char *rows = smem + TABLE_BYTES + ALPHA_BYTES; // row 0 is zero, then the tile
     constexpr int ROW_BYTES = KS * 32 + ROW_PAD;
+    // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows)
+    float *a_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES);
+    float *k_lds = a_lds + max_rows + 1; // K of the tile's pixels, same case
     constexpr int MT = 32 * PS;
     // fragments are fetched in groups of HS steps: half a tap where that is >= 2 steps
     constexpr int HS = (KS % 2 == 0 && KS >= 4) ? KS / 2 : KS;
@@ -178,6 +182,37 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     tile_span(g, tile, MT, lo, hi);
     const int nrows = min(hi - lo + 1, max_rows);
 
+    // ---- the 32*PS output pixels of the tile, one per lane and 32-pixel block -----------------
+    bool live[PS];
+    // Per pixel: LDS address of the row of tap (0,0), and which kernel rows / columns fall
+    // inside the image (bit kh of rowmask, bit kw of colmask; no bits for a dead pixel).
+    uint32_t base_addr[PS], rowmask[PS], colmask[PS];
+    int in0[PS]; // input pixel of tap (0,0), relative to the first staged row
+    uint32_t pix[PS], img[PS], rem[PS];
+#pragma unroll
+    for (int ps = 0; ps < PS; ps++) {
+        pix[ps] = p_first + ps * 32 + (lane & 31);
+        live[ps] = pix[ps] < g.npix_out;
+        const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
+        img[ps] = g.div_ohw.div(pc);
+        rem[ps] = pc - img[ps] * g.ohw;
+        const int oh = (int)g.div_ow.div(rem[ps]);
+        const int ow = (int)rem[ps] - oh * g.ow;
+        in0[ps] = (int)(img[ps] * g.ihw) + (oh - g.ph) * g.iw + (ow - g.pw) - lo;
+        base_addr[ps] = (uint32_t)(size_t)rows + (uint32_t)((1 + in0[ps]) * ROW_BYTES)
+            + (lane >> 5) * 16;
+        // kernel rows kh with 0 <= oh - ph + kh < ih, as a run of bits (kh < 32)
+        auto run_of_bits = [](int first, int last) -> uint32_t { // bits first..last, clipped
+            if (first < 0) first = 0;
+            if (last > 31) last = 31;
+            if (last < first) return 0u;
+            return (uint32_t)(((1ull << (last + 1)) - 1) & ~((1ull << first) - 1));
+        };
+        rowmask[ps] = live[ps] ? run_of_bits(g.ph - oh, g.ih - 1 + g.ph - oh) : 0u;
+        colmask[ps] = run_of_bits(g.pw - ow, g.iw - 1 + g.pw - ow);
+    }
+    const uint32_t zero_addr = (uint32_t)(size_t)rows + (lane >> 5) * 16;
+
     // ---- LDS: lookup table, zero row, this workgroup's alphas, FP4 rows ----------------------
     // The rows of the tile are contiguous in the packed input: item i is word i of that
     // run.  The first EARLY loads of every thread are in flight while the table is built.
@@ -192,11 +227,19 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const int i = u * 256 + tid;
         early[u] = i < nitems ? run[i] : 0u;
     }
+    const bool fuse_k = !RAW && a_plane != nullptr; // uniform
+    float a_early = 0.f;
+    if (fuse_k && tid < nrows) a_early = a_plane[lo + tid];
     table[tid] = fp4_of_byte(tid);
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
     {
         const int oc = chunk * NT + tid;
         alpha_lds[tid] = oc < g.oc ? alpha[oc] : 0.f;
+    }
+    if (fuse_k) { // mean|x| of the staged input pixels, plus one slot that holds zero
+        if (tid < nrows) a_lds[tid] = a_early;
+        if (tid == 0) a_lds[max_rows] = 0.f;
+        for (int i = 256 + tid; i < nrows; i += 256) a_lds[i] = a_plane[lo + i];
     }
     __syncthreads();
     auto expand = [&](int i, uint32_t word) { // item i of the run -> 32 FP4 codes of its row
@@ -212,6 +255,40 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     for (int u = 0; u < EARLY; u++) {
         const int i = u * 256 + tid;
         if (i < nitems) expand(i, early[u]);
+    }
+    // K of the tile's pixels, when it is not read from the K plane: wave ps sums the block
+    // of 32 pixels ps exactly as the box filter does (in-bounds taps in row-major order, each
+    // product rounded, then added: reference src/bcast_calculate_k.cpp:69-85), leaves it in
+    // LDS for the epilogue of all waves and stores it to the K plane.
+    if (fuse_k) {
+#pragma unroll
+        for (int ps = 0; ps < PS; ps++) {
+            if (ps != wave) continue; // uniform
+            float sum = 0.f;
+            // Four taps per round, all reads of a round issued before its first addition.  A
+            // tap outside the image (or past the kernel row) reads the slot that holds zero
+            // and so contributes +0, which leaves the sum of non-negative terms unchanged
+            // bit for bit; reading unconditionally keeps the reads free of branches.
+            for (int kh = 0; kh < g.kh; kh++)
+                for (int kw0 = 0; kw0 < g.kw; kw0 += 4) {
+                    float term[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const int kw = kw0 + u;
+                        const int kwc = kw < g.kw ? kw : 0;
+                        const bool ok = kw < g.kw
+                            && ((rowmask[ps] >> kh) & (colmask[ps] >> kwc) & 1u);
+                        term[u] = __fmul_rn(
+                                a_lds[ok ? in0[ps] + kh * g.iw + kw : max_rows], inv_khw);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) sum = __fadd_rn(sum, term[u]);
+                }
+            if (lane < 32) {
+                k_lds[ps * 32 + lane] = sum;
+                if (chunk == 0 && live[ps]) k_out[pix[ps]] = sum;
+            }
+        }
     }
     for (int base = EARLY * 256; base < nitems; base += 4 * 256) {
         uint32_t w[4];
@@ -230,34 +307,6 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // ---- this wave: 64 filters x 32*PS pixels --------------------------------------------------
     const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
     const bool wave_has_filters = oc_sub0 * 32 < g.oc; // wave-uniform
-    bool live[PS];
-    // Per pixel: LDS address of the row of tap (0,0), and which kernel rows / columns fall
-    // inside the image (bit kh of rowmask, bit kw of colmask; no bits for a dead pixel).
-    uint32_t base_addr[PS], rowmask[PS], colmask[PS];
-    uint32_t pix[PS], img[PS], rem[PS];
-#pragma unroll
-    for (int ps = 0; ps < PS; ps++) {
-        pix[ps] = p_first + ps * 32 + (lane & 31);
-        live[ps] = pix[ps] < g.npix_out;
-        const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
-        img[ps] = g.div_ohw.div(pc);
-        rem[ps] = pc - img[ps] * g.ohw;
-        const int oh = (int)g.div_ow.div(rem[ps]);
-        const int ow = (int)rem[ps] - oh * g.ow;
-        const int in0 = (int)(img[ps] * g.ihw) + (oh - g.ph) * g.iw + (ow - g.pw) - lo;
-        base_addr[ps] = (uint32_t)(size_t)rows + (uint32_t)((1 + in0) * ROW_BYTES)
-            + (lane >> 5) * 16;
-        // kernel rows kh with 0 <= oh - ph + kh < ih, as a run of bits (kh < 32)
-        auto run_of_bits = [](int first, int last) -> uint32_t { // bits first..last, clipped
-            if (first < 0) first = 0;
-            if (last > 31) last = 31;
-            if (last < first) return 0u;
-            return (uint32_t)(((1ull << (last + 1)) - 1) & ~((1ull << first) - 1));
-        };
-        rowmask[ps] = live[ps] ? run_of_bits(g.ph - oh, g.ih - 1 + g.ph - oh) : 0u;
-        colmask[ps] = run_of_bits(g.pw - ow, g.iw - 1 + g.pw - ow);
-    }
-    const uint32_t zero_addr = (uint32_t)(size_t)rows + (lane >> 5) * 16;
 
     v16f acc[2][PS];
 #pragma unroll
@@ -361,6 +410,11 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         advance_tap();
     }
     __syncthreads(); // FP4 rows are in place
+    float kv[PS]; // K of this wave's pixels
+#pragma unroll
+    for (int ps = 0; ps < PS; ps++)
+        kv[ps] = RAW ? 0.f : fuse_k ? k_lds[ps * 32 + (lane & 31)]
+                                    : kplane[live[ps] ? pix[ps] : 0];
     if (wave_has_filters) {
         fetch_rows_after<PS>(b0, rowaddr, acc);
         wait_all_after<PS>(acc);
@@ -390,12 +444,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     auto store_tile = [&](auto check_filters) {
         constexpr bool CHECK = decltype(check_filters)::value;
         int n[PS];
-        float kv[PS];
         size_t nchw0[PS];
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
             n[ps] = opc[rem[ps]];
-            kv[ps] = RAW ? 0.f : kplane[live[ps] ? pix[ps] : 0];
             nchw0[ps] = ((size_t)img[ps] * g.oc) * g.ohw + rem[ps];
         }
         // 64-pixel addressing of the joined blocks: pair q covers pixels 64q + lane
@@ -518,8 +570,9 @@ int max_tile_rows(const Geometry &g, uint32_t mt) {
 }
 
 size_t lds_bytes(const Geometry &g, int ps) {
-    return TABLE_BYTES + ALPHA_BYTES
-        + (size_t)(1 + max_tile_rows(g, 32 * ps)) * (steps_per_tap(g) * 32 + ROW_PAD);
+    const size_t rows = (size_t)max_tile_rows(g, 32 * ps);
+    return TABLE_BYTES + ALPHA_BYTES + (1 + rows) * (steps_per_tap(g) * 32 + ROW_PAD)
+        + (rows + 1 + 32 * ps) * sizeof(float);
 }
 
 // 32-pixel blocks per tile: the choice that minimises (waves on the busiest SIMD) x (work
@@ -548,7 +601,7 @@ int pick_ps(const Geometry &g) {
 template <int KS, int PS>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
-        hipStream_t s) {
+        const float *a_or_null, float *k_out, hipStream_t s) {
     const int chunks = (g.oc + NT - 1) / NT;
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
     const uint32_t units = tiles * chunks, per_xcd = (units + 7) / 8;
@@ -559,22 +612,22 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true>), grid, block, lds, s, xbits,
                 wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw));
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false>), grid, block, lds, s, xbits,
                 wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw));
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
     return hipGetLastError();
 }
 
 template <int KS>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
-        hipStream_t s) {
+        const float *a_or_null, float *k_out, hipStream_t s) {
     switch (g.mfma_ps) {
-    case 2: return launch_mfma<KS, 2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 3: return launch_mfma<KS, 3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 4: return launch_mfma<KS, 4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 2: return launch_mfma<KS, 2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma<KS, 3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 4: return launch_mfma<KS, 4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }
@@ -615,14 +668,14 @@ const char *mfma_kernel_name(const Geometry &g) {
 
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
-        float *dst, int32_t *popc, hipStream_t s) {
+        float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s) {
     switch (steps_per_tap(g)) {
-    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
-    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, s);
+    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }

@@ -69,6 +69,12 @@ struct State {
     // pass over the input when it is called next with the same src and a buffers.
     const void *a_ready_src = nullptr;
     const void *a_ready_buf = nullptr;
+    // K owed: calculate_k has mean|x| in k_owed_a and has not run the box filter, because
+    // the matrix-core convolution computes K from mean|x| on the fly (and stores it to
+    // k_owed_k).  Anything else that needs the K plane, or that is about to overwrite
+    // mean|x|, runs the box filter first (settle_k in api.hip).
+    const float *k_owed_a = nullptr;
+    float *k_owed_k = nullptr;
     bool verbose = false;
 };
 
@@ -93,9 +99,12 @@ const char *mfma_kernel_name(const Geometry &g);
 size_t mfma_weight_bytes(const Geometry &g);
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
         hipStream_t s);
+// With a_or_null set, the kernel ignores k, computes the K plane itself from mean|x| (the
+// box filter of stage 2) and also stores it to k_out.
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
-        float *dst, int32_t *popc_or_null, hipStream_t s);
+        float *dst, int32_t *popc_or_null, const float *a_or_null, float *k_out,
+        hipStream_t s);
 const char *convolution_kernel_name(const Geometry &g);
 const char *binarize_kernel_name(const Geometry &g);
 
