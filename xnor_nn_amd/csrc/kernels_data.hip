@@ -23,26 +23,29 @@ __device__ __forceinline__ uint32_t top_bits(int n) {
     return n >= 32 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu >> n);
 }
 
-// NCHW input.  One workgroup = 64 consecutive pixels of the flattened (mb, ih, iw) index;
-// wave w of the group owns S consecutive 32-channel slices per round (slices
-// (r*NW + w)*S .. +S-1 in round r).  A lane is a pixel, so every load instruction reads 64
-// consecutive floats of one channel plane.  All 32*S loads of a wave are issued before
-// the first use.  Sign bits are shifted into the lane's word with one funnel shift per
-// element (a ballot would produce pixel-major masks of one channel, i.e. the transpose
-// of what is stored).
+// NCHW input.  A tile is 64 consecutive pixels of the flattened (mb, ih, iw) index; wave w of
+// the workgroup owns the 32-channel slices w, w + NW, ... of it.  A lane is a pixel, so every
+// load instruction reads 64 consecutive floats of one channel plane.  All 32 loads of a slice
+// are issued before the first use.  Sign bits are shifted into the lane's word with one
+// funnel shift per element (a ballot would produce pixel-major masks of one channel, i.e.
+// the transpose of what is stored).
 //
 // mean|x| must be summed over channels in order.  The waves therefore hand the running
 // sum from one to the next through LDS: wave w adds its terms after wave w-1 has published
-// its result.  The loads of every wave are in flight during that chain.
+// its result.  The packed words of the tile are staged in LDS and written as one
+// contiguous run.
 //
-// The packed words of the tile are staged in LDS and written as one contiguous run.
+// One workgroup per tile.  (A persistent grid that issues the loads of its next tile before
+// it processes the current one was measured and is not used: at these sizes the kernel is
+// bound by the transfer plus one pass of the sum through the waves, and the hardware's own
+// workgroup scheduling does as well as the hand-made pipeline.)
 //
-// Workgroup b works on tile (b % 8) * tiles_per_xcd + b / 8: workgroups are dealt to the
-// eight XCDs round-robin, so this gives each XCD one contiguous range of tiles and the
-// cache lines that straddle two neighbouring tiles (a channel plane is rarely a multiple
-// of 128 bytes) are fetched into one L2 instead of two.
-template <int S, bool WRITE_BITS, bool WRITE_A>
-__global__ __launch_bounds__(TILE * MAX_WAVES / S)
+// Workgroups are dealt to the eight XCDs round-robin.  XCD x owns the contiguous range of
+// tiles [x * tiles_per_xcd, (x+1) * tiles_per_xcd): the cache lines that straddle two
+// neighbouring tiles (a channel plane is rarely a multiple of 128 bytes) are fetched into
+// one L2 instead of two.  Workgroup b takes local tile b / 8 of XCD b % 8.
+template <bool WRITE_BITS, bool WRITE_A>
+__global__ __launch_bounds__(TILE * MAX_WAVES)
 void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
         float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
         const uint32_t ntiles, const uint32_t tiles_per_xcd) {
@@ -50,69 +53,84 @@ void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bi
     float *chain = reinterpret_cast<float *>(lds); // [TILE]
     uint32_t *stage = lds + TILE;                  // [TILE][xw]
 
-    const uint32_t tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
-    if (tile >= ntiles) return;
-
     const int lane = threadIdx.x & (TILE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nw = blockDim.x >> 6;
+    const uint32_t tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= ntiles) return;
 
-    const uint32_t p = tile * TILE + lane;
-    const bool live = p < g.npix_in;
-    const uint32_t pc = live ? p : g.npix_in - 1;
-    const uint32_t img = g.div_ihw.div(pc);
-    const uint32_t hw = pc - img * g.ihw;
-    const float *base = x + (size_t)img * g.ic * g.ihw + hw;
+    // the whole input as one raw buffer (the host side checks that it is below 4 GiB)
+    const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(x), 0, (int)((uint32_t)g.npix_in * (uint32_t)g.ic * 4u),
+            0x00020000);
+    // slice (r * nw + wave) of a tile: 32 channel values of this lane's pixel
+    auto load_slice = [&](float (&t)[32], uint32_t tile, int r) {
+        const uint32_t p = tile * TILE + lane;
+        const uint32_t pc = p < g.npix_in ? p : g.npix_in - 1;
+        const uint32_t img = g.div_ihw.div(pc);
+        const uint32_t hw = pc - img * g.ihw;
+        const int c0 = (r * nw + wave) * 32; // wave-uniform
+        if (c0 >= g.ic) return;
+        // Buffer loads: one VGPR holds the lane's byte offset for all 32 loads, the channel
+        // plane is a scalar offset (no 64-bit address arithmetic per load, fewer VGPRs).
+        const uint32_t lane_off = (img * (uint32_t)(g.ic * g.ihw) + hw) * 4u;
+        const uint32_t plane_bytes = (uint32_t)g.ihw * 4u;
+        if (c0 + 32 <= g.ic) {
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                t[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        src, lane_off, (uint32_t)(c0 + i) * plane_bytes, 0));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                t[i] = (c0 + i < g.ic)
+                    ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                              src, lane_off, (uint32_t)(c0 + i) * plane_bytes, 0))
+                    : 0.f;
+        }
+    };
 
-    if (wave == 0) chain[lane] = 0.f;
-
-    for (int r = 0; r < rounds; r++) {
-        const int slice0 = (r * nw + wave) * S; // wave-uniform
-        const int c0 = slice0 * 32;
-        const bool has = c0 < g.ic;
-        float t[32 * S];
-        if (has) {
-            const float *col = base + (size_t)c0 * g.ihw;
-            if (c0 + 32 * S <= g.ic) {
-#pragma unroll
-                for (int i = 0; i < 32 * S; i++) t[i] = col[(size_t)i * g.ihw];
-            } else {
-#pragma unroll
-                for (int i = 0; i < 32 * S; i++)
-                    t[i] = (c0 + i < g.ic) ? col[(size_t)i * g.ihw] : 0.f;
-            }
-#pragma unroll
-            for (int sl = 0; sl < S; sl++) {
+    // everything after the loads of round 0; t holds them on entry
+    auto process = [&](float (&t)[32], uint32_t tile) {
+        const uint32_t p = tile * TILE + lane;
+        if (wave == 0) chain[lane] = 0.f;
+        for (int r = 0; r < rounds; r++) {
+            if (r > 0) load_slice(t, tile, r);
+            const int slice = r * nw + wave; // wave-uniform
+            const int c0 = slice * 32;
+            const bool has = c0 < g.ic;
+            if (has) {
                 uint32_t neg = 0; // sign bits, first channel ends up in the MSB
 #pragma unroll
                 for (int i = 0; i < 32; i++) {
-                    neg = __builtin_amdgcn_alignbit(neg, fbits(t[32 * sl + i]), 31);
-                    t[32 * sl + i] = __fmul_rn(__builtin_fabsf(t[32 * sl + i]), inv_ic);
+                    neg = __builtin_amdgcn_alignbit(neg, fbits(t[i]), 31);
+                    t[i] = __fmul_rn(__builtin_fabsf(t[i]), inv_ic);
                 }
-                const int n = g.ic - (c0 + 32 * sl);
-                if (WRITE_BITS && n > 0)
-                    stage[lane * g.xw + slice0 + sl] = (~neg) & top_bits(n);
+                if (WRITE_BITS) stage[lane * g.xw + slice] = (~neg) & top_bits(g.ic - c0);
             }
-        }
-        // ordered hand-over of the running sum: wave s goes after wave s-1
-        for (int s = 0; s < nw; s++) {
-            if (s == wave && has) {
-                float acc = chain[lane];
+            // ordered hand-over of the running sum: wave s goes after wave s-1
+            for (int s = 0; s < nw; s++) {
+                if (s == wave && has) {
+                    float acc = chain[lane];
 #pragma unroll
-                for (int i = 0; i < 32 * S; i++) acc = __fadd_rn(acc, t[i]);
-                chain[lane] = acc;
+                    for (int i = 0; i < 32; i++) acc = __fadd_rn(acc, t[i]);
+                    chain[lane] = acc;
+                }
+                __syncthreads();
             }
-            __syncthreads();
         }
-    }
+        const size_t tile_words = (size_t)TILE * g.xw;
+        const size_t first = (size_t)tile * tile_words;
+        const size_t total = (size_t)g.npix_in * g.xw;
+        if (WRITE_BITS)
+            for (uint32_t i = threadIdx.x; i < tile_words; i += blockDim.x)
+                if (first + i < total) bits[first + i] = stage[i];
+        if (WRITE_A && wave == 0 && p < g.npix_in) a[p] = chain[lane];
+    };
 
-    const size_t tile_words = (size_t)TILE * g.xw;
-    const size_t first = (size_t)tile * tile_words;
-    const size_t total = (size_t)g.npix_in * g.xw;
-    if (WRITE_BITS)
-        for (uint32_t i = threadIdx.x; i < tile_words; i += blockDim.x)
-            if (first + i < total) bits[first + i] = stage[i];
-    if (WRITE_A && wave == 0 && live) a[p] = chain[lane];
+    float t[32];
+    load_slice(t, tile, 0);
+    process(t, tile);
 }
 
 // Any source layout, one lane per pixel, channels visited in order.  Used for NHWC input
@@ -173,45 +191,34 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
     k[p] = acc;
 }
 
-// Slices per wave.  Two slices per wave halve the waves of a workgroup but need over 100
-// VGPRs, which leaves no more workgroups resident than one slice per wave does; measured
-// equal or slower on MI355X, so one is used.
-int slices_per_wave(const Geometry &g) {
-    if (const char *e = getenv("XNOR_NN_HIP_BIN_S")) return atoi(e) == 2 ? 2 : 1;
-    (void)g;
-    return 1;
-}
-
-template <int S, bool WRITE_BITS, bool WRITE_A>
+template <bool WRITE_BITS, bool WRITE_A>
 void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
-    const int max_waves = MAX_WAVES / S;
-    const int need = (g.xw + S - 1) / S;
-    const int nw = need < max_waves ? need : max_waves;
+    const int need = g.xw;
+    const int nw = need < MAX_WAVES ? need : MAX_WAVES;
     const int rounds = (need + nw - 1) / nw;
     const uint32_t ntiles = (g.npix_in + TILE - 1) / TILE;
     const uint32_t per_xcd = (ntiles + 7) / 8;
     const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
-    hipLaunchKernelGGL((binarize_nchw_kernel<S, WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
+    hipLaunchKernelGGL((binarize_nchw_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
             dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
-}
-
-template <bool WRITE_BITS, bool WRITE_A>
-void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
-    if (slices_per_wave(g) == 2) launch_nchw<2, WRITE_BITS, WRITE_A>(g, x, bits, a, s);
-    else launch_nchw<1, WRITE_BITS, WRITE_A>(g, x, bits, a, s);
 }
 
 } // namespace
 
+// The tiled kernel addresses the input with 32-bit byte offsets.
+static bool tiled_nchw(const Geometry &g) {
+    return g.src_fmt == xnor_nn_data_format_nchw
+        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull;
+}
+
 const char *binarize_kernel_name(const Geometry &g) {
-    return g.src_fmt == xnor_nn_data_format_nchw ? "binarize_nchw_kernel"
-                                                 : "binarize_generic_kernel";
+    return tiled_nchw(g) ? "binarize_nchw_kernel" : "binarize_generic_kernel";
 }
 
 hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
         float *a_or_null, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
-    if (g.src_fmt == xnor_nn_data_format_nchw) {
+    if (tiled_nchw(g)) {
         if (a_or_null) launch_nchw<true, true>(g, x, bits, a_or_null, s);
         else launch_nchw<true, false>(g, x, bits, nullptr, s);
     } else {
@@ -228,7 +235,7 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
 
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
-    if (g.src_fmt == xnor_nn_data_format_nchw) {
+    if (tiled_nchw(g)) {
         launch_nchw<false, true>(g, x, nullptr, a, s);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
