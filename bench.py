@@ -22,7 +22,11 @@ MFMA_FP4_PEAK_TOPS = 10100.0
 # HBM bytes per launch read from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch),
 # each scaled by what the same counter shows for a plain copy of known size; the runs and
 # the scale factors are recorded in profiles/.  Not measurable from inside this script.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # profiles/alexnet_conv4_mb256_hbm_traffic_pmc.txt: read (FETCH_SIZE x2) + written bytes
+    ("alexnet_conv4_mb256", "conv_mfma_fp4_kernel"): 6102 * 1024 + 43880 * 1024,
+    ("alexnet_conv4_mb256", "binarize_nchw_kernel"): 65720 * 1024 + 2197 * 1024,
+}
 
 
 def work_figures(d):
@@ -198,7 +202,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u32 xnor/popcount, int32 accumulate, fp32 scale",
+        "dtype": ("fp4 (E2M1, +-1 exactly) MFMA, fp32 accumulate (exact integers), fp32 scale"
+                  if on_mfma else "u32 xnor/popcount, int32 accumulate, fp32 scale"),
         "data": "synthetic (hash-based N(0,1)/N(0,sigma), seeds 1234/4321), resident in HBM",
         "config": {"workload": args.workload,
                    "shape": {k: d[k] for k in ("mb", "ic", "ih", "iw", "oc", "kh", "kw",
