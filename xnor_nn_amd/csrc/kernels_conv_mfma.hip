@@ -39,6 +39,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int NT = 256;       // filters per workgroup (4 waves x 64)
 constexpr int ROW_PAD = 16;   // spare bytes per LDS row
@@ -434,81 +435,94 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     }
 
     // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
-    //      pixel lane%32.  Values are scaled in that layout; then v_permlane32_swap joins two
-    //      pixel blocks, so that a register holds 64 consecutive pixels of ONE filter and a
-    //      store instruction writes one 256-byte run of the NCHW output (the odd block of
-    //      PS = 3 keeps the 2 x 128-byte form).  The runs of one filter are stored back to
-    //      back so that the cache lines they share fill up in L2 before they can leave it. ----
+    //      pixel lane%32.  Values are scaled in that layout.  For NCHW output
+    //      v_permlane32_swap then joins two pixel blocks, so that a register holds 64
+    //      consecutive pixels of ONE filter and a store instruction writes one 256-byte run
+    //      (the odd block of PS = 3 keeps the 2 x 128-byte form); the runs of one filter are
+    //      stored back to back so that the cache lines they share fill up in L2 before they
+    //      can leave it.  Stores are raw buffer stores: the lane's pixel offset is one VGPR
+    //      computed once, the filter is a scalar offset, and a dead pixel or a filter past
+    //      OC gets an offset beyond the buffer, which the hardware drops; no 64-bit address
+    //      arithmetic and no branches per store. ------------------------------------------------
     if (!wave_has_filters) return;
     const int lane_hi = lane >> 5;
-    auto store_tile = [&](auto check_filters) {
-        constexpr bool CHECK = decltype(check_filters)::value;
-        int n[PS];
-        size_t nchw0[PS];
+    constexpr uint32_t DROP = 0xFFFFFFF0u; // >= the buffer size: the store is discarded
+    const __amdgpu_buffer_rsrc_t outbuf = __builtin_amdgcn_make_buffer_rsrc(
+            RAW ? static_cast<void *>(popc) : static_cast<void *>(dst), 0,
+            (int)((uint32_t)g.npix_out * (uint32_t)g.oc * 4u), 0x00020000);
+    const bool nchw = RAW || g.dst_fmt == xnor_nn_data_format_nchw;
+    const uint32_t fstep = nchw ? (uint32_t)g.ohw * 4u : 4u; // bytes from a filter to the next
+    int n[PS];
+    uint32_t off1[PS]; // one block: lanes 0..31 filter f, lanes 32..63 filter f + 4
 #pragma unroll
-        for (int ps = 0; ps < PS; ps++) {
-            n[ps] = opc[rem[ps]];
-            nchw0[ps] = ((size_t)img[ps] * g.oc) * g.ohw + rem[ps];
-        }
-        // 64-pixel addressing of the joined blocks: pair q covers pixels 64q + lane
-        bool live64[PS / 2 > 0 ? PS / 2 : 1];
-        size_t at64[PS / 2 > 0 ? PS / 2 : 1];
+    for (int ps = 0; ps < PS; ps++) {
+        n[ps] = RAW ? opc[rem[ps]] : 0;
+        const uint32_t at = nchw ? (img[ps] * (uint32_t)g.oc * (uint32_t)g.ohw + rem[ps]) * 4u
+                                 : pix[ps] * (uint32_t)g.oc * 4u;
+        off1[ps] = live[ps] ? at + (uint32_t)lane_hi * 4u * fstep : DROP;
+    }
+    uint32_t off2[PS / 2 > 0 ? PS / 2 : 1]; // joined pair q: pixels 64q + lane of one filter
 #pragma unroll
-        for (int q = 0; q < PS / 2; q++) {
-            const uint32_t p64 = p_first + q * 64 + lane;
-            live64[q] = p64 < g.npix_out;
-            const uint32_t pc = live64[q] ? p64 : g.npix_out - 1;
-            const uint32_t im = g.div_ohw.div(pc);
-            at64[q] = ((size_t)im * g.oc) * g.ohw + (pc - im * g.ohw);
-        }
-        const bool joined = RAW || g.dst_fmt == xnor_nn_data_format_nchw;
+    for (int q = 0; q < PS / 2; q++) {
+        const uint32_t p64 = p_first + q * 64 + lane;
+        const uint32_t pc = p64 < g.npix_out ? p64 : g.npix_out - 1;
+        const uint32_t im = g.div_ohw.div(pc);
+        off2[q] = p64 < g.npix_out
+            ? (im * (uint32_t)g.oc * (uint32_t)g.ohw + (pc - im * g.ohw)) * 4u : DROP;
+    }
+    auto store_tile = [&](auto check_filters, auto planar) {
+        constexpr bool CHECK = decltype(check_filters)::value, NCHW = decltype(planar)::value;
 #pragma unroll
         for (int os = 0; os < 2; os++) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int oc_lo = (wave * 2 + os) * 32 + 8 * (i / 4) + (i & 3); // lanes 0..31
-                const int ocl = oc_lo + lane_hi * 4;
-                const int oc = chunk * NT + ocl;
-                uint32_t v[PS]; // bit patterns of the results in the accumulator layout
+            for (int i4 = 0; i4 < 4; i4++) {
+                // alphas of the four filters 8*i4 + 4*lane_hi + 0..3 of this 32-filter block
+                const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
+                const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
 #pragma unroll
-                for (int ps = 0; ps < PS; ps++) {
-                    const float d = acc[os][ps][i]; // = 2*popc - n, exactly
-                    if constexpr (RAW)
-                        v[ps] = (uint32_t)(((int)d + n[ps]) / 2);
-                    else // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
-                        v[ps] = __float_as_uint(__fmul_rn(__fmul_rn(d, alpha_lds[ocl]), kv[ps]));
-                }
-                uint32_t *out = RAW ? reinterpret_cast<uint32_t *>(popc)
-                                    : reinterpret_cast<uint32_t *>(dst);
-                if (joined) {
+                for (int ii = 0; ii < 4; ii++) {
+                    const int i = 4 * i4 + ii;
+                    const int f = chunk * NT + (wave * 2 + os) * 32 + 8 * i4 + ii; // lanes 0..31
+                    const uint32_t soff = (uint32_t)f * fstep; // uniform
+                    uint32_t v[PS]; // bit patterns of the results in the accumulator layout
 #pragma unroll
-                    for (int q = 0; q < PS / 2; q++) {
-                        const auto r = __builtin_amdgcn_permlane32_swap(v[2 * q], v[2 * q + 1],
-                                false, false);
-                        // r[0]: filter oc_lo, pixels 64q + lane; r[1]: filter oc_lo + 4
-                        const int oc_a = chunk * NT + oc_lo, oc_b = oc_a + 4;
-                        if (live64[q] && !(CHECK && oc_a >= g.oc))
-                            out[at64[q] + (size_t)oc_a * g.ohw] = r[0];
-                        if (live64[q] && !(CHECK && oc_b >= g.oc))
-                            out[at64[q] + (size_t)oc_b * g.ohw] = r[1];
+                    for (int ps = 0; ps < PS; ps++) {
+                        const float d = acc[os][ps][i]; // = 2*popc - n, exactly
+                        if constexpr (RAW)
+                            v[ps] = (uint32_t)(((int)d + n[ps]) / 2);
+                        else // dst = fl(fl((float)(2*popc - n) * alpha) * k), rounded per product
+                            v[ps] = __float_as_uint(__fmul_rn(__fmul_rn(d, al[ii]), kv[ps]));
                     }
-                    if constexpr (PS % 2 == 1) {
-                        if (live[PS - 1] && !(CHECK && oc >= g.oc))
-                            out[nchw0[PS - 1] + (size_t)oc * g.ohw] = v[PS - 1];
-                    }
-                } else {
+                    if constexpr (NCHW) {
 #pragma unroll
-                    for (int ps = 0; ps < PS; ps++)
-                        if (live[ps] && !(CHECK && oc >= g.oc))
-                            out[(size_t)pix[ps] * g.oc + oc] = v[ps];
+                        for (int q = 0; q < PS / 2; q++) {
+                            const auto r = __builtin_amdgcn_permlane32_swap(v[2 * q],
+                                    v[2 * q + 1], false, false);
+                            // r[0]: filter f, pixels 64q + lane; r[1]: filter f + 4
+                            if (!CHECK || f < g.oc)
+                                __builtin_amdgcn_raw_buffer_store_b32(r[0], outbuf, off2[q], soff, 0);
+                            if (!CHECK || f + 4 < g.oc)
+                                __builtin_amdgcn_raw_buffer_store_b32(r[1], outbuf, off2[q],
+                                        soff + 4u * fstep, 0);
+                        }
+                    }
+#pragma unroll
+                    for (int ps = NCHW ? (PS / 2) * 2 : 0; ps < PS; ps++) {
+                        const uint32_t voff = CHECK && f + lane_hi * 4 >= g.oc ? DROP : off1[ps];
+                        __builtin_amdgcn_raw_buffer_store_b32(v[ps], outbuf, voff, soff, 0);
+                    }
                 }
             }
         }
     };
-    if (chunk * NT + (wave + 1) * 64 <= g.oc) // wave-uniform: all 64 filters exist
-        store_tile(std::false_type{});
-    else
-        store_tile(std::true_type{});
+    const bool all_filters = chunk * NT + (wave + 1) * 64 <= g.oc; // wave-uniform
+    if (nchw) {
+        if (all_filters) store_tile(std::false_type{}, std::true_type{});
+        else store_tile(std::true_type{}, std::true_type{});
+    } else {
+        if (all_filters) store_tile(std::false_type{}, std::false_type{});
+        else store_tile(std::true_type{}, std::false_type{});
+    }
 }
 
 // One thread per dword of the fragment layout [OC/32][tap][KS][lane][4 dwords]:
@@ -575,8 +589,13 @@ size_t lds_bytes(const Geometry &g, int ps) {
         + (rows + 1 + 32 * ps) * sizeof(float);
 }
 
-// 32-pixel blocks per tile: the choice that minimises (waves on the busiest SIMD) x (work
-// per wave); ties go to the larger tile, which streams fewer weight bytes.
+// 32-pixel blocks per tile.  Cost of a choice = (waves the busiest SIMD runs one after the
+// other) x (work per wave, plus half a block for the staging and epilogue every tile pays).
+// With few waves per SIMD the busiest one sets the pace, so the count is rounded up; with
+// many, the hardware's dynamic scheduling evens the load out.  Ties go to the larger tile,
+// which streams fewer weight bytes.  (Measured on MI355X: conv4 MB 256 PS 2/3/4 = 29.1 /
+// 28.5 / 32.2 us, ResNet 3x3 MB 64 = 87.3 / 90.7 / 83.2, VGG 512 MB 32 = 42.6 / 46.1 / 39.3,
+// conv2 shape MB 128 = 54.1 / 51.3 / 49.7.)
 int pick_ps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
         const int v = atoi(e);
@@ -591,8 +610,9 @@ int pick_ps(const Geometry &g) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
-        const double busiest = per_simd <= 1 ? 1 : (double)(long)(per_simd + 0.999999);
-        const double cost = busiest * ps;
+        const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
+                                             : per_simd + 0.5;
+        const double cost = (busiest < 1 ? 1 : busiest) * (ps + 0.5);
         if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
     }
     return best;
@@ -644,6 +664,7 @@ int mfma_tile_blocks(const Geometry &g) {
     if (g.sh != 1 || g.sw != 1) return 0;
     if ((g.ic + 63) / 64 > 8) return 0;
     if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
+    if ((uint64_t)g.npix_out * g.oc * 4u >= 0xFFFFFFF0ull) return 0; // 32-bit output offsets
     if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
     return pick_ps(g);
 }
