@@ -56,9 +56,9 @@ __host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, uint
     uint32_t p_last = p_first + mt;
     if (p_last > g.npix_out) p_last = g.npix_out;
     p_last -= 1;
-    const uint32_t i0 = p_first / g.ohw, i1 = p_last / g.ohw;
-    const int oh0 = (int)((p_first - i0 * g.ohw) / g.ow);
-    const int oh1 = (int)((p_last - i1 * g.ohw) / g.ow);
+    const uint32_t i0 = g.div_ohw.div(p_first), i1 = g.div_ohw.div(p_last);
+    const int oh0 = (int)g.div_ow.div(p_first - i0 * g.ohw);
+    const int oh1 = (int)g.div_ow.div(p_last - i1 * g.ohw);
     int r0 = oh0 - g.ph, r1 = oh1 - g.ph + g.kh - 1;
     if (r0 < 0) r0 = 0;
     if (r0 > g.ih - 1) r0 = g.ih - 1;
@@ -176,7 +176,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // share and the output cache lines they both write into meet in one L2.
     const uint32_t unit = (blockIdx.x & 7) * units_per_xcd + (blockIdx.x >> 3);
     if (unit >= units) return;
-    const uint32_t tile = unit / oc_chunks;
+    const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
     const int chunk = unit - tile * oc_chunks;
     const int taps = g.kh * g.kw;
 

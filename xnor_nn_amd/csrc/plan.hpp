@@ -27,8 +27,12 @@ struct FastDiv {
         f.sh2 = L - 1;
         return f;
     }
-    __device__ __forceinline__ uint32_t div(uint32_t n) const {
-        uint32_t t = __umulhi(n, mul);
+    __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        const uint32_t t = __umulhi(n, mul);
+#else
+        const uint32_t t = (uint32_t)(((uint64_t)n * mul) >> 32);
+#endif
         return (t + ((n - t) >> sh1)) >> sh2;
     }
 };
