@@ -5,6 +5,8 @@ Bar: packed tensors, operation counts and integer popcount accumulators bit-exac
 float tensors (a, k, alpha, dst) are computed in the reference's summation order and are
 asserted bit-exact as well, which is stricter than the 1e-5 relative tolerance allowed for
 them (the tolerance check is kept in `check_floats` for the error message only)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -217,6 +219,23 @@ def test_calculate_k_alone_matches_fused_path(oracle, gpu):
     conv.stage("calculate_k", src=xt)
     assert np.array_equal(conv.export_floats(capi.RES_K), k_want)
     conv.close()
+
+
+@pytest.mark.parametrize("exe", ["simple_convolution_c", "simple_convolution_cpp"])
+def test_upstream_example_programs_run_unchanged(gpu, exe):
+    """The reference's own example programs (reference example/simple_convolution.c and
+    .cpp: host buffers, algorithm "best", three forward passes), compiled unchanged against
+    include/ and linked to this library by `make -C oracle examples`, run to completion.
+    The C program prints the status string of its last call."""
+    import subprocess
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "oracle", "_ref", "examples", exe)
+    if not os.path.exists(path):
+        pytest.skip("example programs not built (upstream sources were not mounted)")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, (out.stdout, out.stderr)
+    if exe.endswith("_c"):
+        assert out.stdout.strip() == "success"
 
 
 def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
