@@ -43,7 +43,7 @@ void pack_weights_kernel(const float *__restrict__ w, uint32_t *__restrict__ bit
 }
 
 // alpha[oc] = sum over (ic, kh, kw), nested in that order, of fl(|w| * chw)
-// (reference src/bcast_binarize_weights.cpp:95-115).  One thread per filter.
+// (reference src/bcast_binarize_weights.cpp:95-115).  One thread per filter, any layout.
 __global__ __launch_bounds__(64)
 void alpha_kernel(const float *__restrict__ w, float *__restrict__ alpha,
         const Geometry g, const float chw) {
@@ -56,6 +56,64 @@ void alpha_kernel(const float *__restrict__ w, float *__restrict__ alpha,
                 acc = __fadd_rn(acc,
                         __fmul_rn(__builtin_fabsf(w[w_index(g, oc, ic, kh, kw)]), chw));
     alpha[oc] = acc;
+}
+
+// The same sum for OIHW weights, where a filter is one contiguous row of n = IC*KH*KW floats
+// already in summation order.  One wave per ALPHA_F filters.  The rows are read ALPHA_CHUNK
+// elements at a time with coalesced loads (all lanes read consecutive elements of one
+// filter), passed through LDS and summed in order by lane f for filter f; the loads of the
+// next chunk are in flight while the current one is summed.  Few filters per wave and long
+// chunks: the sum is a serial chain either way, and this shape keeps many bytes in flight
+// per wave and spreads the filters over many CUs.
+constexpr int ALPHA_F = 8;
+constexpr int ALPHA_CHUNK = 512;
+
+__global__ __launch_bounds__(64)
+void alpha_oihw_kernel(const float *__restrict__ w, float *__restrict__ alpha, const int oc_n,
+        const int n, const float chw) {
+    __shared__ float tile[ALPHA_F][ALPHA_CHUNK + 1];
+    constexpr int PER_LANE = ALPHA_CHUNK / 64;
+    const int lane = threadIdx.x;
+    const int f0 = blockIdx.x * ALPHA_F;
+    const int nf = min(ALPHA_F, oc_n - f0);
+    float acc = 0.f;
+    float cur[ALPHA_F][PER_LANE], nxt[ALPHA_F][PER_LANE]; // element c0 + 64*u + lane of filter f
+    auto fetch = [&](float (&v)[ALPHA_F][PER_LANE], int c0) {
+#pragma unroll
+        for (int f = 0; f < ALPHA_F; f++)
+#pragma unroll
+            for (int u = 0; u < PER_LANE; u++) {
+                const int e = c0 + 64 * u + lane;
+                v[f][u] = (f < nf && e < n) ? w[(size_t)(f0 + f) * n + e] : 0.f;
+            }
+    };
+    fetch(cur, 0);
+    for (int c0 = 0; c0 < n; c0 += ALPHA_CHUNK) {
+        if (c0 + ALPHA_CHUNK < n) fetch(nxt, c0 + ALPHA_CHUNK);
+#pragma unroll
+        for (int f = 0; f < ALPHA_F; f++)
+#pragma unroll
+            for (int u = 0; u < PER_LANE; u++)
+                tile[f][64 * u + lane] = __fmul_rn(__builtin_fabsf(cur[f][u]), chw);
+        __syncthreads();
+        // Elements past the end of the row were stored as +0, and s + 0 == s for these
+        // non-negative sums, so whole batches can be read before they are added in order.
+        if (lane < ALPHA_F) {
+            for (int j = 0; j < ALPHA_CHUNK; j += 16) {
+                float v[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) v[u] = tile[lane][j + u];
+#pragma unroll
+                for (int u = 0; u < 16; u++) acc = __fadd_rn(acc, v[u]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < ALPHA_F; f++)
+#pragma unroll
+            for (int u = 0; u < PER_LANE; u++) cur[f][u] = nxt[f][u];
+    }
+    if (lane < nf) alpha[f0 + lane] = acc;
 }
 
 // opc[oh][ow] = IC * number of in-bounds taps (reference
@@ -111,7 +169,12 @@ hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *
     hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256),
             0, s, w, bits, g);
     const float chw = 1.f / (g.ic * g.kh * g.kw);
-    hipLaunchKernelGGL(alpha_kernel, dim3((g.oc + 63) / 64), dim3(64), 0, s, w, alpha, g, chw);
+    if (g.w_fmt == xnor_nn_weights_format_oihw)
+        hipLaunchKernelGGL(alpha_oihw_kernel, dim3((g.oc + ALPHA_F - 1) / ALPHA_F), dim3(64), 0,
+                s, w, alpha,
+                g.oc, g.ic * g.kh * g.kw, chw);
+    else
+        hipLaunchKernelGGL(alpha_kernel, dim3((g.oc + 63) / 64), dim3(64), 0, s, w, alpha, g, chw);
     hipLaunchKernelGGL(op_count_kernel, dim3((g.ohw + 255) / 256), dim3(256), 0, s, opc, g);
     return hipGetLastError();
 }
