@@ -125,7 +125,11 @@ def test_workloads_full_size_digests(oracle, golden, gpu, name):
     (capi.FMT_NHWC, capi.FMT_HWIO, capi.FMT_NHWC),
 ])
 @pytest.mark.parametrize("t", [(3, 40, 32, 9, 11, 3, 3, 1, 1, 1, 1),
-                               (2, 96, 48, 13, 13, 5, 5, 1, 1, 2, 2)], ids=shapes.shape_id)
+                               (2, 96, 48, 13, 13, 5, 5, 1, 1, 2, 2),
+                               # full 64-filter waves (16-byte NHWC stores), IC = 3 words + 4
+                               (3, 256, 100, 13, 13, 3, 3, 1, 1, 1, 1),
+                               # IC not a multiple of 4: the generic NHWC kernel
+                               (1, 12, 37, 6, 7, 3, 3, 1, 1, 1, 1)], ids=shapes.shape_id)
 def test_tensor_formats(oracle, fmts, t):
     """NHWC input, HWIO weights and NHWC output (reference
     src/bcast_binarize_data.cpp:56-57, src/bcast_binarize_weights.cpp:71-72,

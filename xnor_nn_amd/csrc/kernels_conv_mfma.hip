@@ -473,6 +473,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         off2[q] = p64 < g.npix_out
             ? (im * (uint32_t)g.oc * (uint32_t)g.ohw + (pc - im * g.ohw)) * 4u : DROP;
     }
+    // 16-byte stores need filter runs that start on a 16-byte boundary
+    const bool vec4_ok = !nchw && (g.oc & 3) == 0
+        && ((size_t)(RAW ? static_cast<void *>(popc) : static_cast<void *>(dst)) & 15) == 0;
     auto store_tile = [&](auto check_filters, auto planar) {
         constexpr bool CHECK = decltype(check_filters)::value, NCHW = decltype(planar)::value;
 #pragma unroll
@@ -482,6 +485,28 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                 // alphas of the four filters 8*i4 + 4*lane_hi + 0..3 of this 32-filter block
                 const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
                 const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
+                if constexpr (!NCHW && !CHECK) {
+                    // NHWC: registers 4*i4 .. +3 are four consecutive filters of the lane's
+                    // pixel, i.e. 16 contiguous bytes; the two lane halves write 32 and
+                    // the wave's eight stores per pixel block fill 256 bytes of each pixel.
+                    if (vec4_ok) {
+                        const uint32_t soff = (uint32_t)(chunk * NT + (wave * 2 + os) * 32
+                                + 8 * i4) * 4u;
+#pragma unroll
+                        for (int ps = 0; ps < PS; ps++) {
+                            v4i q;
+#pragma unroll
+                            for (int ii = 0; ii < 4; ii++) {
+                                const float d = acc[os][ps][4 * i4 + ii];
+                                q[ii] = RAW ? (((int)d + n[ps]) / 2)
+                                            : (int)__float_as_uint(__fmul_rn(
+                                                      __fmul_rn(d, al[ii]), kv[ps]));
+                            }
+                            __builtin_amdgcn_raw_buffer_store_b128(q, outbuf, off1[ps], soff, 0);
+                        }
+                        continue;
+                    }
+                }
 #pragma unroll
                 for (int ii = 0; ii < 4; ii++) {
                     const int i = 4 * i4 + ii;

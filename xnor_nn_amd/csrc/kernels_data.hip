@@ -166,6 +166,70 @@ void binarize_generic_kernel(const float *__restrict__ x, uint32_t *__restrict__
     if (WRITE_A) a[p] = acc;
 }
 
+// NHWC input with IC a multiple of 4: a lane is a pixel and walks over its channels, which
+// are contiguous, in order, 32 at a time (one packed word): eight 16-byte buffer loads per
+// word, the loads of the next three words in flight while the current one is folded into
+// the sign word and the running mean|x| (reference src/bcast_binarize_data.cpp:56-57,
+// src/bcast_calculate_k.cpp:59-60).  The lanes of a wave read addresses IC*4 bytes apart,
+// so every load touches 64 cache lines, but each line is used completely by the loads that
+// follow, and HBM traffic is the algorithmic minimum.
+template <bool WRITE_BITS, bool WRITE_A>
+__global__ __launch_bounds__(256)
+void binarize_nhwc_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
+        float *__restrict__ a, const Geometry g, const float inv_ic) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t pc = p < g.npix_in ? p : g.npix_in - 1;
+    const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(x), 0, (int)((uint32_t)g.npix_in * (uint32_t)g.ic * 4u),
+            0x00020000);
+    const uint32_t lane_off = pc * (uint32_t)g.ic * 4u;
+    // 32 channels starting at c0; channels >= IC read as +0 (sign bit clear, |x| = 0: they
+    // are masked out of the word and add nothing to the sum)
+    auto fetch = [&](v4f (&v)[8], int c0) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int c = c0 + 4 * u; // uniform
+            v[u] = c < g.ic ? __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                                      src, lane_off, (uint32_t)c * 4u, 0))
+                            : v4f{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    float acc = 0.f;
+    auto fold = [&](const v4f (&v)[8], int j) { // word j: sign bits and the running sum
+        if (j >= g.xw) return; // uniform
+        uint32_t neg = 0; // sign bits, first channel ends up in the MSB
+        const int n = min(32, g.ic - 32 * j);
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float val = v[u][e];
+                neg = __builtin_amdgcn_alignbit(neg, fbits(val), 31);
+                if (4 * u + e < n) // uniform; a sum must not see the padding's +0 terms
+                    acc = __fadd_rn(acc, __fmul_rn(__builtin_fabsf(val), inv_ic));
+            }
+        if (WRITE_BITS && p < g.npix_in) bits[(size_t)p * g.xw + j] = (~neg) & top_bits(n);
+    };
+    // four register sets used in turn: three words are in flight while one is folded
+    v4f b0[8], b1[8], b2[8], b3[8];
+    fetch(b0, 0);
+    fetch(b1, 32);
+    fetch(b2, 64);
+    for (int j = 0; j < g.xw; j += 4) {
+        fetch(b3, 32 * (j + 3));
+        fold(b0, j);
+        fetch(b0, 32 * (j + 4));
+        fold(b1, j + 1);
+        fetch(b1, 32 * (j + 5));
+        fold(b2, j + 2);
+        fetch(b2, 32 * (j + 6));
+        fold(b3, j + 3);
+    }
+    if (WRITE_A && p < g.npix_in) a[p] = acc;
+}
+
 // K plane: k = sum over in-bounds taps, row-major, of fl(a * KHW)
 // (reference src/bcast_calculate_k.cpp:69-85).  One lane per output pixel.
 __global__ __launch_bounds__(256)
@@ -211,8 +275,15 @@ static bool tiled_nchw(const Geometry &g) {
         && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull;
 }
 
+// The NHWC kernel reads 16 bytes per load at 32-bit byte offsets.
+static bool vector_nhwc(const Geometry &g) {
+    return g.src_fmt == xnor_nn_data_format_nhwc && (g.ic & 3) == 0
+        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull;
+}
+
 const char *binarize_kernel_name(const Geometry &g) {
-    return tiled_nchw(g) ? "binarize_nchw_kernel" : "binarize_generic_kernel";
+    return tiled_nchw(g) ? "binarize_nchw_kernel"
+        : vector_nhwc(g) ? "binarize_nhwc_kernel" : "binarize_generic_kernel";
 }
 
 hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
@@ -221,6 +292,14 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
     if (tiled_nchw(g)) {
         if (a_or_null) launch_nchw<true, true>(g, x, bits, a_or_null, s);
         else launch_nchw<true, false>(g, x, bits, nullptr, s);
+    } else if (vector_nhwc(g)) {
+        const unsigned blocks = (g.npix_in + 255) / 256;
+        if (a_or_null)
+            hipLaunchKernelGGL((binarize_nhwc_kernel<true, true>), dim3(blocks), dim3(256), 0,
+                    s, x, bits, a_or_null, g, inv_ic);
+        else
+            hipLaunchKernelGGL((binarize_nhwc_kernel<true, false>), dim3(blocks), dim3(256), 0,
+                    s, x, bits, a_or_null, g, inv_ic);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
         if (a_or_null)
@@ -237,6 +316,10 @@ hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStrea
     const float inv_ic = 1.f / g.ic;
     if (tiled_nchw(g)) {
         launch_nchw<false, true>(g, x, nullptr, a, s);
+    } else if (vector_nhwc(g)) {
+        const unsigned blocks = (g.npix_in + 255) / 256;
+        hipLaunchKernelGGL((binarize_nhwc_kernel<false, true>), dim3(blocks), dim3(256), 0, s,
+                x, nullptr, a, g, inv_ic);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
         hipLaunchKernelGGL((binarize_generic_kernel<false, true>), dim3(blocks), dim3(256),
