@@ -194,6 +194,35 @@ def test_popcount_kernel_still_matches(oracle, gpu, monkeypatch):
         conv_name = make(d, w).kernel_name(0)
         assert conv_name.startswith("conv_xnor_popc"), conv_name
         run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+    # strides above 1, ragged channel and filter counts
+    for t in ((1, 70, 20, 7, 5, 3, 3, 2, 2, 1, 1), (1, 24, 16, 12, 12, 7, 7, 3, 3, 3, 3),
+              (2, 96, 64, 28, 28, 3, 3, 2, 2, 1, 1)):
+        d = shapes.as_dims(t)
+        x = synth.normal(51, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+            d["mb"], d["ic"], d["ih"], d["iw"])
+        w = synth.normal(52, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+            d["oc"], d["ic"], d["kh"], d["kw"])
+        run_and_compare(oracle, d, x, w)
+
+
+@pytest.mark.parametrize("t", [
+    (2, 96, 64, 28, 28, 3, 3, 2, 2, 1, 1),     # ResNet-style 3x3 stride 2
+    (3, 128, 64, 28, 28, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2 shortcut
+    (2, 64, 96, 27, 27, 5, 5, 2, 2, 2, 2),     # 5x5 stride 2, ragged channels
+    (1, 32, 130, 31, 29, 3, 3, 3, 2, 1, 1),    # different strides per axis
+    (2, 64, 64, 23, 23, 7, 7, 4, 4, 2, 2),     # 7x7 stride 4
+], ids=shapes.shape_id)
+def test_strided_shapes_on_the_matrix_core_kernel(oracle, t):
+    """Strides above 1 run the matrix-core kernel too (the staged span of input pixels then
+    also holds the ones the stride skips)."""
+    d = shapes.as_dims(t)
+    x = synth.normal(61, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(62, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    conv_name = make(d, w).kernel_name(0)
+    assert conv_name.startswith("conv_mfma"), conv_name
+    run_and_compare(oracle, d, x, w)
 
 
 def test_known_answer_forward_on_gpu():

@@ -48,8 +48,9 @@ constexpr int ALPHA_BYTES = NT * 4;
 constexpr int LDS_LIMIT = 64 * 1024;
 
 // First and last input pixel (flattened index) that the tile of mt output pixels starting
-// at tile*mt can touch with an in-bounds tap, for stride 1: from the start of the first
-// input row of its first pixel to the end of the last input row of its last pixel.
+// at tile*mt can touch with an in-bounds tap: from the start of the first input row of its
+// first pixel to the end of the last input row of its last pixel (with a stride above 1
+// the span also holds the input pixels the stride skips).
 __host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, uint32_t mt,
         int &lo, int &hi) {
     const uint32_t p_first = tile * mt;
@@ -59,7 +60,7 @@ __host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, uint
     const uint32_t i0 = g.div_ohw.div(p_first), i1 = g.div_ohw.div(p_last);
     const int oh0 = (int)g.div_ow.div(p_first - i0 * g.ohw);
     const int oh1 = (int)g.div_ow.div(p_last - i1 * g.ohw);
-    int r0 = oh0 - g.ph, r1 = oh1 - g.ph + g.kh - 1;
+    int r0 = oh0 * g.sh - g.ph, r1 = oh1 * g.sh - g.ph + g.kh - 1;
     if (r0 < 0) r0 = 0;
     if (r0 > g.ih - 1) r0 = g.ih - 1;
     if (r1 > g.ih - 1) r1 = g.ih - 1;
@@ -180,7 +181,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const int chunk = unit - tile * oc_chunks;
     const int taps = g.kh * g.kw;
 
-    // ---- which input pixels does the tile touch (stride 1) ----------------------------
+    // ---- which input pixels does the tile touch ------------------------------------------
     const uint32_t p_first = tile * MT;
     int lo, hi;
     tile_span(g, tile, MT, lo, hi);
@@ -202,18 +203,19 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         rem[ps] = pc - img[ps] * g.ohw;
         const int oh = (int)g.div_ow.div(rem[ps]);
         const int ow = (int)rem[ps] - oh * g.ow;
-        in0[ps] = (int)(img[ps] * g.ihw) + (oh - g.ph) * g.iw + (ow - g.pw) - lo;
+        const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw; // input pixel of tap (0,0)
+        in0[ps] = (int)(img[ps] * g.ihw) + ih0 * g.iw + iw0 - lo;
         base_addr[ps] = (uint32_t)(size_t)rows + (uint32_t)((1 + in0[ps]) * ROW_BYTES)
             + (lane >> 5) * 16;
-        // kernel rows kh with 0 <= oh - ph + kh < ih, as a run of bits (kh < 32)
+        // kernel rows kh with 0 <= ih0 + kh < ih, as a run of bits (kh < 32)
         auto run_of_bits = [](int first, int last) -> uint32_t { // bits first..last, clipped
             if (first < 0) first = 0;
             if (last > 31) last = 31;
             if (last < first) return 0u;
             return (uint32_t)(((1ull << (last + 1)) - 1) & ~((1ull << first) - 1));
         };
-        rowmask[ps] = live[ps] ? run_of_bits(g.ph - oh, g.ih - 1 + g.ph - oh) : 0u;
-        colmask[ps] = run_of_bits(g.pw - ow, g.iw - 1 + g.pw - ow);
+        rowmask[ps] = live[ps] ? run_of_bits(-ih0, g.ih - 1 - ih0) : 0u;
+        colmask[ps] = run_of_bits(-iw0, g.iw - 1 - iw0);
     }
     const uint32_t zero_addr = (uint32_t)(size_t)rows + (lane >> 5) * 16;
 
@@ -682,14 +684,13 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 
 } // namespace
 
-// The matrix-core kernel covers stride-1 convolutions with up to 512 input channels whose
+// The matrix-core kernel covers convolutions with up to 512 input channels whose
 // tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
 // Returns the tile size (32-pixel blocks per workgroup, 2..4) or 0 when not applicable.
 int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
         if (e[0] == 'v') return 0;
-    if (g.sh != 1 || g.sw != 1) return 0;
     if ((g.ic + 63) / 64 > 8) return 0;
     if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
     if ((uint64_t)g.npix_out * g.oc * 4u >= 0xFFFFFFF0ull) return 0; // 32-bit output offsets
