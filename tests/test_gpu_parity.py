@@ -175,7 +175,7 @@ def test_edge_shapes(oracle, t):
     run_and_compare(oracle, d, x, w)
 
 
-@pytest.mark.parametrize("ps", ["2", "3", "4"])
+@pytest.mark.parametrize("ps", ["1", "2", "3", "4"])
 def test_matrix_core_tile_sizes(oracle, gpu, monkeypatch, ps):
     """Every tile size of the matrix-core kernel on a workload whose last tile is ragged."""
     monkeypatch.setenv("XNOR_NN_HIP_MFMA_PS", ps)

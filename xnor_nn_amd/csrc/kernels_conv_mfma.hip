@@ -24,7 +24,7 @@
 //     per step feed 2*PS matrix instructions: with PS >= 3 the weight stream stays well
 //     below what the vector memory path of a compute unit delivers (with 2 x 2 blocking it
 //     ran at 80% of it and set the pace).
-//   * PS (2, 3 or 4) is chosen per problem so that the waves divide evenly over the SIMDs:
+//   * PS (1 to 4) is chosen per problem so that the waves divide evenly over the SIMDs:
 //     for 43264 pixels, PS = 3 gives 1.76 waves per SIMD (2 in the busiest), PS = 4 gives
 //     1.32 (also 2, but each a third longer).
 #include <cstdlib>
@@ -97,6 +97,7 @@ __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c)
 __device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src));
 }
+#define XNOR_ACC1 "+v"(acc[0][0]), "+v"(acc[1][0])
 #define XNOR_ACC2 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1])
 #define XNOR_ACC3 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[1][0]), \
         "+v"(acc[1][1]), "+v"(acc[1][2])
@@ -104,14 +105,19 @@ __device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
         "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3])
 template <int PS>
 __device__ __forceinline__ void wait_all_after(v16f (&acc)[2][PS]) {
-    if constexpr (PS == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC2);
+    if constexpr (PS == 1) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC1);
+    else if constexpr (PS == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC2);
     else if constexpr (PS == 3) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC3);
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC4);
 }
 template <int PS>
 __device__ __forceinline__ void fetch_rows_after(v4i (&bn)[PS], const uint32_t (&a)[PS],
         v16f (&acc)[2][PS]) {
-    if constexpr (PS == 2)
+    if constexpr (PS == 1)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]"
+                : [b0] "=&v"(bn[0]), XNOR_ACC1
+                : [a0] "v"(a[0]));
+    else if constexpr (PS == 2)
         asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
                      "ds_read_b128 %[b1], %[a1]"
                 : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), XNOR_ACC2
@@ -129,6 +135,7 @@ __device__ __forceinline__ void fetch_rows_after(v4i (&bn)[PS], const uint32_t (
                   XNOR_ACC4
                 : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]));
 }
+#undef XNOR_ACC1
 #undef XNOR_ACC2
 #undef XNOR_ACC3
 #undef XNOR_ACC4
@@ -629,14 +636,14 @@ size_t lds_bytes(const Geometry &g, int ps) {
 int pick_ps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
         const int v = atoi(e);
-        if (v >= 2 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT) return v;
+        if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT) return v;
     }
     const int chunks = (g.oc + NT - 1) / NT;
     const int waves_per_block = g.oc >= NT ? 4 : (g.oc + 63) / 64;
     const double simds = (double)g.cus * 4;
     int best = 0;
     double best_cost = 0;
-    for (int ps = 4; ps >= 2; ps--) {
+    for (int ps = 4; ps >= 1; ps--) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
@@ -675,6 +682,7 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
     switch (g.mfma_ps) {
+    case 1: return launch_mfma<KS, 1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 2: return launch_mfma<KS, 2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 3: return launch_mfma<KS, 3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 4: return launch_mfma<KS, 4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
@@ -687,7 +695,7 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 // The matrix-core kernel covers convolutions with up to 512 input channels whose
 // tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
-// Returns the tile size (32-pixel blocks per workgroup, 2..4) or 0 when not applicable.
+// Returns the tile size (32-pixel blocks per workgroup, 1..4) or 0 when not applicable.
 int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
         if (e[0] == 'v') return 0;

@@ -58,7 +58,7 @@ struct Geometry {
     uint32_t npix_in, npix_out; // mb*ihw, mb*ohw
     int cus;                    // compute units of the device (256 if it cannot be asked)
     int use_mfma;               // 1: stage 3 runs the FP4 matrix-core kernel
-    int mfma_ps;                // its tile size in 32-pixel blocks (2..4)
+    int mfma_ps;                // its tile size in 32-pixel blocks (1..4)
     size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
