@@ -14,7 +14,7 @@ namespace xnor_hip {
 namespace {
 
 constexpr int TILE = 64;       // pixels per workgroup = lanes per wave
-constexpr int MAX_WAVES = 16;  // 1024 threads
+constexpr int MAX_WAVES = 8;   // waves per workgroup
 
 __device__ __forceinline__ uint32_t fbits(float v) { return __float_as_uint(v); }
 
@@ -257,9 +257,12 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
 
 template <bool WRITE_BITS, bool WRITE_A>
 void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
+    // At most eight waves per workgroup, the slices split evenly over the rounds: with more
+    // waves the hand-over chain of one workgroup gets long and too few workgroups are
+    // resident to cover it (512 input channels: 14.1 us with 16 waves, 10.4 us with 2 x 8).
     const int need = g.xw;
-    const int nw = need < MAX_WAVES ? need : MAX_WAVES;
-    const int rounds = (need + nw - 1) / nw;
+    const int rounds = (need + MAX_WAVES - 1) / MAX_WAVES;
+    const int nw = (need + rounds - 1) / rounds;
     const uint32_t ntiles = (g.npix_in + TILE - 1) / TILE;
     const uint32_t per_xcd = (ntiles + 7) / 8;
     const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
