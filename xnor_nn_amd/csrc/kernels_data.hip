@@ -14,7 +14,7 @@ namespace xnor_hip {
 namespace {
 
 constexpr int TILE = 64;       // pixels per workgroup = lanes per wave
-constexpr int MAX_WAVES = 8;   // waves per workgroup
+constexpr int MAX_WAVES = 12;  // waves per workgroup
 
 __device__ __forceinline__ uint32_t fbits(float v) { return __float_as_uint(v); }
 
@@ -45,7 +45,7 @@ __device__ __forceinline__ uint32_t top_bits(int n) {
 // neighbouring tiles (a channel plane is rarely a multiple of 128 bytes) are fetched into
 // one L2 instead of two.  Workgroup b takes local tile b / 8 of XCD b % 8.
 template <bool WRITE_BITS, bool WRITE_A>
-__global__ __launch_bounds__(TILE * MAX_WAVES)
+__global__ __launch_bounds__(TILE * 16)
 void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
         float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
         const uint32_t ntiles, const uint32_t tiles_per_xcd) {
@@ -257,11 +257,18 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
 
 template <bool WRITE_BITS, bool WRITE_A>
 void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
-    // At most eight waves per workgroup, the slices split evenly over the rounds: with more
+    // At most twelve waves per workgroup, the slices split evenly over the rounds: with more
     // waves the hand-over chain of one workgroup gets long and too few workgroups are
-    // resident to cover it (512 input channels: 14.1 us with 16 waves, 10.4 us with 2 x 8).
+    // resident to cover it (512 input channels: 14.1 us with 16 waves, 10.4 us with 2 x 8;
+    // 384 channels: 12 x 1 and 6 x 2 are equal at MB 256, 12 x 1 is 5% faster at MB 1024).
+    // XNOR_NN_HIP_BIN_WAVES overrides the cap for measurements.
     const int need = g.xw;
-    const int rounds = (need + MAX_WAVES - 1) / MAX_WAVES;
+    int cap = MAX_WAVES;
+    if (const char *e = getenv("XNOR_NN_HIP_BIN_WAVES")) {
+        const int v = atoi(e);
+        if (v >= 1 && v <= 16) cap = v;
+    }
+    const int rounds = (need + cap - 1) / cap;
     const int nw = (need + rounds - 1) / rounds;
     const uint32_t ntiles = (g.npix_in + TILE - 1) / TILE;
     const uint32_t per_xcd = (ntiles + 7) / 8;
