@@ -139,7 +139,8 @@ def main():
     wt = torch.from_numpy(w).to(dev)
     yt = torch.empty((d["mb"], d["oc"], wf["oh"], wf["ow"]), dtype=torch.float32, device=dev)
 
-    stream = torch.cuda.current_stream()
+    # a stream of its own: the legacy default stream synchronises implicitly with others
+    stream = torch.cuda.Stream()
     conv = Convolution(capi.ALGORITHM_BCAST, capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW,
                        d["mb"], d["oc"], d["ic"], d["ih"], d["iw"], d["kh"], d["kw"],
                        d["sh"], d["sw"], d["ph"], d["pw"], wt, stream=stream)
@@ -158,6 +159,7 @@ def main():
         if events:
             events[3].record(stream)
 
+    torch.cuda.synchronize()  # inputs were written on the default stream
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -225,6 +225,51 @@ def test_strided_shapes_on_the_matrix_core_kernel(oracle, t):
     run_and_compare(oracle, d, x, w)
 
 
+def test_forward_pass_captured_in_a_hip_graph(oracle, gpu):
+    """The three executors enqueue kernels only (no allocation, no memset, no host
+    synchronisation when the tensors are on the device), so a caller may capture them in a
+    HIP graph.  Every replay, with eager passes and synchronisations in between, must give
+    the eager result bit for bit."""
+    import torch
+    d, x, w = synth.make_workload("alexnet_conv4_mb256", 24)
+    x2 = np.ascontiguousarray(x[::-1])
+    s = oracle_shape(oracle, d)
+    want, want2 = oracle.forward(s, x, w)["dst"], oracle.forward(s, x2, w)["dst"]
+    side = torch.cuda.Stream()
+    xt = torch.from_numpy(x).to(gpu)
+    x2t = torch.from_numpy(x2).to(gpu)
+    yt = torch.empty(want.shape, dtype=torch.float32, device=gpu)
+    conv = make(d, torch.from_numpy(w).to(gpu))
+    conv.set_stream(side)
+
+    def step():
+        conv.stage("binarize_data", src=xt, dst=yt)
+        conv.stage("calculate_k")
+        conv.stage("forward")
+
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        step() # eager pass first: the staging state of the descriptor is settled
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    for i in range(4):
+        yt.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(yt.cpu().numpy().view(np.uint32), want.view(np.uint32)), i
+        # eager work of the same descriptor on other data between the replays
+        with torch.cuda.stream(side):
+            conv.stage("binarize_data", src=x2t, dst=yt)
+            conv.stage("calculate_k")
+            conv.stage("forward")
+        side.synchronize()
+        assert np.array_equal(yt.cpu().numpy().view(np.uint32), want2.view(np.uint32)), i
+    conv.close()
+
+
 def test_known_answer_forward_on_gpu():
     """The reference's 18 precomputed outputs
     (reference test/gtest/test_convolution_reference_forward.cpp:20-73), tolerance 1e-3."""
