@@ -225,6 +225,53 @@ def test_strided_shapes_on_the_matrix_core_kernel(oracle, t):
     run_and_compare(oracle, d, x, w)
 
 
+def _random_case(rng):
+    kh, kw = int(rng.integers(1, 8)), int(rng.integers(1, 8))
+    ph, pw = int(rng.integers(0, 4)), int(rng.integers(0, 4))
+    sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    # the reference derives oh AND ow from pw, so keep both extents consistent with that
+    ih = int(rng.integers(max(1, kh - 2 * pw), 22))
+    iw = int(rng.integers(max(1, kw - 2 * pw), 22))
+    ic = int(rng.choice([1, 3, 31, 32, 33, 64, 65, 96, 100, 128, 160, 200, 257]))
+    oc = int(rng.choice([1, 7, 16, 31, 32, 33, 64, 65, 100, 130, 256, 260]))
+    mb = int(rng.integers(1, 5))
+    fmts = (int(rng.choice([capi.FMT_NCHW, capi.FMT_NHWC])),
+            int(rng.choice([capi.FMT_OIHW, capi.FMT_HWIO])),
+            int(rng.choice([capi.FMT_NCHW, capi.FMT_NHWC])))
+    return (mb, ic, oc, ih, iw, kh, kw, sh, sw, ph, pw), fmts
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_strides_and_layouts(oracle, seed):
+    """Seeded random problems (channel counts around the 32/64 boundaries, kernels 1..7,
+    strides 1..3, paddings 0..3, all layout combinations), ten per seed, every intermediate
+    against the oracle.  Inputs carry exact zeros of both signs."""
+    rng = np.random.default_rng(1000 + seed)
+    done = 0
+    while done < 10:
+        t, fmts = _random_case(rng)
+        d = shapes.as_dims(t)
+        oh = (d["ih"] + 2 * d["pw"] - d["kh"]) // d["sh"] + 1
+        ow = (d["iw"] + 2 * d["pw"] - d["kw"]) // d["sw"] + 1
+        if oh < 1 or ow < 1 or d["ih"] + 2 * d["ph"] < d["kh"]:
+            continue
+        x = synth.normal(7000 + 100 * seed + done, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+            d["mb"], d["ic"], d["ih"], d["iw"])
+        x.ravel()[::7] = 0.0
+        x.ravel()[3::11] = -0.0
+        w = synth.normal(9000 + 100 * seed + done, d["oc"] * d["ic"] * d["kh"] * d["kw"],
+                         0.05).reshape(d["oc"], d["ic"], d["kh"], d["kw"])
+        if fmts[0] == capi.FMT_NHWC:
+            x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+        if fmts[1] == capi.FMT_HWIO:
+            w = np.ascontiguousarray(w.transpose(2, 3, 1, 0))
+        try:
+            run_and_compare(oracle, d, x, w, fmts)
+        except AssertionError as e:
+            raise AssertionError("case %s formats %s: %s" % (shapes.shape_id(t), fmts, e))
+        done += 1
+
+
 def test_forward_pass_captured_in_a_hip_graph(oracle, gpu):
     """The three executors enqueue kernels only (no allocation, no memset, no host
     synchronisation when the tensors are on the device), so a caller may capture them in a
