@@ -178,7 +178,6 @@ __global__ __launch_bounds__(256)
 void binarize_nhwc_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
         float *__restrict__ a, const Geometry g, const float inv_ic) {
     typedef float v4f __attribute__((ext_vector_type(4)));
-    typedef int v4i __attribute__((ext_vector_type(4)));
     const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t pc = p < g.npix_in ? p : g.npix_in - 1;
     const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(
