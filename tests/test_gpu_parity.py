@@ -161,7 +161,10 @@ def test_tensor_formats(oracle, fmts, t):
     (1, 448, 70, 6, 6, 3, 3, 1, 1, 1, 1),     # 7 steps (run as 8)
     (7, 64, 40, 10, 10, 3, 3, 1, 1, 2, 2),    # padding larger than the usual "same"
     (2, 32, 64, 16, 16, 4, 4, 1, 1, 0, 0),    # even filter size, output smaller than input
-    (1, 640, 32, 5, 5, 3, 3, 1, 1, 1, 1),     # more than 512 channels: popcount kernel
+    (1, 640, 32, 5, 5, 3, 3, 1, 1, 1, 1),     # more than 512 channels: 12 steps, quarter-tap groups
+    (2, 1024, 70, 7, 7, 1, 1, 1, 1, 0, 0),    # 1x1 over 1024 channels: 16 steps
+    (1, 1000, 40, 6, 6, 3, 3, 1, 1, 1, 1),    # 16 steps with a ragged last word, 3x3
+    (3, 768, 260, 9, 9, 3, 3, 2, 2, 1, 1),    # 12 steps, stride 2, more than 256 filters
 ], ids=shapes.shape_id)
 def test_edge_shapes(oracle, t):
     d = shapes.as_dims(t)

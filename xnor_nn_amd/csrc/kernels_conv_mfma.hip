@@ -150,7 +150,8 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
     return out;
 }
 
-// KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4), PS = 32-pixel
+// KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4 and to 12 or 16
+// above 8), PS = 32-pixel
 // blocks per workgroup tile.
 template <int KS, int PS, bool RAW>
 __global__ __launch_bounds__(256, 2)
@@ -173,8 +174,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // the registers allow it (8 VGPRs per step on top of 32 per pixel block), half a tap
     // otherwise.  The longer lead hides more of the L2 latency of the fragment stream
     // (conv4 MB 256: main loop 11.9 -> 10.9 us per wave).
-    constexpr int HS = (KS % 2 == 0 && KS >= 4 && (PS > 3 || 40 * PS + 16 * KS > 216)) ? KS / 2 : KS;
-    constexpr int GROUPS_PER_TAP = KS / HS;
+    // Above 8 steps per tap (more than 512 channels) a group is a quarter of a tap.
+    constexpr int HS = KS > 8 ? KS / 4
+        : (KS % 2 == 0 && KS >= 4 && (PS > 3 || 40 * PS + 16 * KS > 216)) ? KS / 2 : KS;
+    constexpr int GROUPS_PER_TAP = KS / HS; // 1, 2 or 4
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -434,6 +437,21 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         constexpr int P1 = HS & 1, OFF1 = GROUPS_PER_TAP == 2 ? HS * 32 : 0;
         using std::integral_constant;
         int n = 0;
+        if constexpr (GROUPS_PER_TAP == 4) { // the four quarters of a tap, wa and wb in turn
+            for (; n + 3 <= last_group; n += 4) {
+                run_group(std::true_type{}, std::false_type{}, integral_constant<int, 0>{},
+                        integral_constant<int, 0>{}, integral_constant<int, HS * 32>{}, n, wa, wb);
+                run_group(std::true_type{}, std::false_type{}, integral_constant<int, P1>{},
+                        integral_constant<int, HS * 32>{}, integral_constant<int, 2 * HS * 32>{},
+                        n + 1, wb, wa);
+                run_group(std::true_type{}, std::false_type{}, integral_constant<int, 0>{},
+                        integral_constant<int, 2 * HS * 32>{},
+                        integral_constant<int, 3 * HS * 32>{}, n + 2, wa, wb);
+                run_group(std::true_type{}, std::true_type{}, integral_constant<int, P1>{},
+                        integral_constant<int, 3 * HS * 32>{}, integral_constant<int, 0>{},
+                        n + 3, wb, wa);
+            }
+        }
         for (; n + 1 <= last_group; n += 2) {
             run_group(std::true_type{}, integral_constant<bool, GROUPS_PER_TAP == 1>{},
                     integral_constant<int, 0>{}, integral_constant<int, 0>{},
@@ -594,10 +612,11 @@ void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__
     frag[i] = out;
 }
 
-// Steps per tap as the kernel is instantiated: ceil(IC/64), odd counts above 4 rounded up
-// (the extra step multiplies FP4 zeros).
+// Steps per tap as the kernel is instantiated: ceil(IC/64), odd counts above 4 rounded up,
+// counts above 8 rounded up to 12 or 16 (the extra steps multiply FP4 zeros).
 int steps_per_tap(const Geometry &g) {
     const int ks = (g.ic + 63) / 64;
+    if (ks > 8) return (ks + 3) / 4 * 4; // 12 or 16
     return ks > 4 && (ks & 1) ? ks + 1 : ks;
 }
 int oc_subblocks(const Geometry &g) { return ((g.oc + NT - 1) / NT) * (NT / 32); }
@@ -636,7 +655,9 @@ size_t lds_bytes(const Geometry &g, int ps) {
 int pick_ps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
         const int v = atoi(e);
-        if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT) return v;
+        if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT
+                && !(v == 4 && steps_per_tap(g) > 8))
+            return v;
     }
     const int chunks = (g.oc + NT - 1) / NT;
     const int waves_per_block = g.oc >= NT ? 4 : (g.oc + 63) / 64;
@@ -645,6 +666,7 @@ int pick_ps(const Geometry &g) {
     double best_cost = 0;
     for (int ps = 4; ps >= 1; ps--) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
+        if (ps == 4 && steps_per_tap(g) > 8) continue; // would not fit the register file
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
         const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
@@ -692,14 +714,14 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 
 } // namespace
 
-// The matrix-core kernel covers convolutions with up to 512 input channels whose
+// The matrix-core kernel covers convolutions with up to 1024 input channels whose
 // tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
 // Returns the tile size (32-pixel blocks per workgroup, 1..4) or 0 when not applicable.
 int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
         if (e[0] == 'v') return 0;
-    if ((g.ic + 63) / 64 > 8) return 0;
+    if ((g.ic + 63) / 64 > 16) return 0;
     if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
     if ((uint64_t)g.npix_out * g.oc * 4u >= 0xFFFFFFF0ull) return 0; // 32-bit output offsets
     if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
@@ -734,6 +756,8 @@ hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
     case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 12: return launch_mfma_ps<12>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 16: return launch_mfma_ps<16>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }
