@@ -188,6 +188,28 @@ def test_matrix_core_tile_sizes(oracle, gpu, monkeypatch, ps):
     run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
 
 
+@pytest.mark.parametrize("pair", ["0", "1"])
+@pytest.mark.parametrize("t", [
+    (2, 96, 64, 13, 13, 5, 5, 1, 1, 2, 2),     # 3 words, 25 taps (odd: last pair has one tap)
+    (3, 32, 70, 9, 11, 3, 3, 1, 1, 1, 1),      # 1 word: two taps per matrix instruction
+    (1, 20, 33, 8, 8, 2, 2, 1, 1, 0, 0),       # 1 ragged word, even number of taps
+    (2, 160, 40, 10, 10, 3, 3, 2, 2, 1, 1),    # 5 words, stride 2
+    (1, 150, 300, 7, 6, 4, 3, 1, 1, 1, 1),     # 5 words (ragged), more than 256 filters
+], ids=shapes.shape_id)
+def test_tap_pairing(oracle, monkeypatch, t, pair):
+    """Odd numbers of 32-channel words per pixel: the matrix-core kernel with and without
+    two taps sharing their steps (XNOR_NN_HIP_MFMA_PAIR forces either)."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_PAIR", pair)
+    d = shapes.as_dims(t)
+    x = synth.normal(71, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(72, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    name = make(d, w).kernel_name(0)
+    assert name.startswith("conv_mfma") and name.endswith(",PAIR>") == (pair == "1"), name
+    run_and_compare(oracle, d, x, w)
+
+
 def test_popcount_kernel_still_matches(oracle, gpu, monkeypatch):
     """The XNOR/popcount kernel (the general fallback) on shapes the matrix-core kernel
     would otherwise take."""

@@ -153,7 +153,7 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
 // KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4 and to 12 or 16
 // above 8), PS = 32-pixel
 // blocks per workgroup tile.
-template <int KS, int PS, bool RAW>
+template <int KS, int PS, bool RAW, bool PAIR>
 __global__ __launch_bounds__(256, 2)
 void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
@@ -165,7 +165,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
     unsigned char *rows = smem + TABLE_BYTES + ALPHA_BYTES; // row 0 is zero, then the tile
-    constexpr int ROW_BYTES = KS * 32 + ROW_PAD;
+    // PAIR (an odd number KS of 32-channel words per pixel): two taps share KS steps, so no
+    // step is half empty; the rows then hold exactly KS words (16*KS bytes is 4 mod 8 dwords,
+    // which keeps the fragment reads conflict-free without padding).
+    constexpr int ROW_BYTES = PAIR ? KS * 16 : KS * 32 + ROW_PAD;
     // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows)
     float *a_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES);
     float *k_lds = a_lds + max_rows + 1; // K of the tile's pixels, same case
@@ -175,7 +178,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // otherwise.  The longer lead hides more of the L2 latency of the fragment stream
     // (conv4 MB 256: main loop 11.9 -> 10.9 us per wave).
     // Above 8 steps per tap (more than 512 channels) a group is a quarter of a tap.
-    constexpr int HS = KS > 8 ? KS / 4
+    constexpr int HS = PAIR ? KS : KS > 8 ? KS / 4
         : (KS % 2 == 0 && KS >= 4 && (PS > 3 || 40 * PS + 16 * KS > 216)) ? KS / 2 : KS;
     constexpr int GROUPS_PER_TAP = KS / HS; // 1, 2 or 4
 
@@ -189,7 +192,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     if (unit >= units) return;
     const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
     const int chunk = unit - tile * oc_chunks;
-    const int taps = g.kh * g.kw;
+    // "taps" below are the units the main loop walks over: kernel taps, or pairs of them
+    const int taps = PAIR ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
 
     // ---- which input pixels does the tile touch ------------------------------------------
     const uint32_t p_first = tile * MT;
@@ -216,7 +220,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw; // input pixel of tap (0,0)
         in0[ps] = (int)(img[ps] * g.ihw) + ih0 * g.iw + iw0 - lo;
         base_addr[ps] = (uint32_t)(size_t)rows + (uint32_t)((1 + in0[ps]) * ROW_BYTES)
-            + (lane >> 5) * 16;
+            + (PAIR ? 0 : (lane >> 5) * 16);
         // kernel rows kh with 0 <= ih0 + kh < ih, as a run of bits (kh < 32)
         auto run_of_bits = [](int first, int last) -> uint32_t { // bits first..last, clipped
             if (first < 0) first = 0;
@@ -227,7 +231,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         rowmask[ps] = live[ps] ? run_of_bits(-ih0, g.ih - 1 - ih0) : 0u;
         colmask[ps] = run_of_bits(-iw0, g.iw - 1 - iw0);
     }
-    const uint32_t zero_addr = (uint32_t)(size_t)rows + (lane >> 5) * 16;
+    const uint32_t zero_addr = (uint32_t)(size_t)rows + (PAIR ? 0 : (lane >> 5) * 16);
 
     // ---- LDS: lookup table, zero row, this workgroup's alphas, FP4 rows ----------------------
     // The rows of the tile are contiguous in the packed input: item i is word i of that
@@ -358,9 +362,39 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         }
     };
     int nkh = 0, nkw = 0; // the tap after the one being multiplied (the last tap repeats)
+    bool ntap_valid = true; // PAIR: false once the walk has run past the last tap
     auto advance_tap = [&]() {
         if (nkw + 1 < g.kw) nkw++;
         else if (nkh + 1 < g.kh) { nkw = 0; nkh++; }
+        else ntap_valid = false;
+    };
+    // PAIR: rows of the two taps of a pair (index 0 and 1); a missing second tap (odd number
+    // of taps, or the repeated last pair) reads the zero row.
+    auto pair_rows = [&](uint32_t (&out)[2][PS]) {
+        tap_rows(nkh, nkw, out[0]);
+        if (!ntap_valid) {
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) out[0][ps] = zero_addr;
+        }
+        advance_tap();
+        tap_rows(nkh, nkw, out[1]);
+        if (!ntap_valid) {
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) out[1][ps] = zero_addr;
+        }
+        advance_tap();
+    };
+    // PAIR: address of step hs for this lane: lanes 0..31 take word 2*hs, lanes 32..63 word
+    // 2*hs + 1 of the 2*KS words of the pair (first tap's KS words, then the second's)
+    const bool lane_hi_half = lane >= 32;
+    auto pair_addr = [&](int hs, const uint32_t (&r)[2][PS], uint32_t (&out)[PS]) {
+        const int c_lo = 2 * hs, c_hi = 2 * hs + 1;
+#pragma unroll
+        for (int ps = 0; ps < PS; ps++) {
+            const uint32_t lo = c_lo < KS ? r[0][ps] + c_lo * 16 : r[1][ps] + (c_lo - KS) * 16;
+            const uint32_t hi = c_hi < KS ? r[0][ps] + c_hi * 16 : r[1][ps] + (c_hi - KS) * 16;
+            out[ps] = lane_hi_half ? hi : lo;
+        }
     };
     auto mma = [&](const v4i (&w)[2], const v4i (&b)[PS]) {
 #pragma unroll
@@ -371,7 +405,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     };
 
     const int last_group = taps * GROUPS_PER_TAP - 1;
-    uint32_t rowaddr[PS]; // rows of the current group's tap
+    uint32_t rowaddr[PS];                    // rows of the current group's tap
+    uint32_t pairaddr[PAIR ? 2 : 1][PAIR ? PS : 1]; // PAIR: rows of both taps of the pair
     v4i b0[PS], b1[PS];   // pixel fragments of the current and the following step, in turn
     // One group with the fragments in wc, while those of the next group arrive in wn.
     // P0: which of b0/b1 holds the group's first step; OFF / NOFF: byte offset within a row of
@@ -386,9 +421,12 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         constexpr int P0 = decltype(p0)::value, OFF = decltype(off)::value,
                       NOFF = decltype(noff)::value;
         uint32_t nextaddr[PS];
+        uint32_t nextpair[PAIR ? 2 : 1][PAIR ? PS : 1];
         if constexpr (MORE) {
             request(min(n + 1, last_group), wn);
-            if constexpr (NEWTAP) { // the next group starts the next tap
+            if constexpr (PAIR) {
+                pair_rows(nextpair);
+            } else if constexpr (NEWTAP) { // the next group starts the next tap
                 tap_rows(nkh, nkw, nextaddr);
                 advance_tap();
             } else {
@@ -400,10 +438,15 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         for (int hs = 0; hs < HS; hs++) {
             if (hs + 1 < HS || MORE) {
                 uint32_t a[PS];
+                if constexpr (PAIR) {
+                    if (hs + 1 < HS) pair_addr(hs + 1, pairaddr, a);
+                    else pair_addr(0, nextpair, a);
+                } else {
 #pragma unroll
-                for (int ps = 0; ps < PS; ps++)
-                    a[ps] = hs + 1 < HS ? rowaddr[ps] + OFF + (hs + 1) * 32
-                                        : nextaddr[ps] + NOFF;
+                    for (int ps = 0; ps < PS; ps++)
+                        a[ps] = hs + 1 < HS ? rowaddr[ps] + OFF + (hs + 1) * 32
+                                            : nextaddr[ps] + NOFF;
+                }
                 if (((P0 + hs) & 1) == 0) fetch_rows_after<PS>(b1, a, acc);
                 else fetch_rows_after<PS>(b0, a, acc);
             } else {
@@ -414,16 +457,28 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         }
         if constexpr (MORE) {
             wait_all_after<PS>(acc); // wn and the first pixel fragments of the next group are in
+            if constexpr (PAIR) {
 #pragma unroll
-            for (int ps = 0; ps < PS; ps++) rowaddr[ps] = nextaddr[ps];
+                for (int ps = 0; ps < PS; ps++) {
+                    pairaddr[0][ps] = nextpair[0][ps];
+                    pairaddr[1][ps] = nextpair[1][ps];
+                }
+            } else {
+#pragma unroll
+                for (int ps = 0; ps < PS; ps++) rowaddr[ps] = nextaddr[ps];
+            }
         }
     };
 
     v4i wa[HS][2], wb[HS][2];
     if (wave_has_filters) {
         request(0, wa);
-        tap_rows(0, 0, rowaddr);
-        advance_tap();
+        if constexpr (PAIR) {
+            pair_rows(pairaddr);
+        } else {
+            tap_rows(0, 0, rowaddr);
+            advance_tap();
+        }
     }
     __syncthreads(); // FP4 rows are in place
     float kv[PS]; // K of this wave's pixels
@@ -432,7 +487,13 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         kv[ps] = RAW ? 0.f : fuse_k ? k_lds[ps * 32 + (lane & 31)]
                                     : kplane[live[ps] ? pix[ps] : 0];
     if (wave_has_filters) {
-        fetch_rows_after<PS>(b0, rowaddr, acc);
+        if constexpr (PAIR) {
+            uint32_t a0[PS];
+            pair_addr(0, pairaddr, a0);
+            fetch_rows_after<PS>(b0, a0, acc);
+        } else {
+            fetch_rows_after<PS>(b0, rowaddr, acc);
+        }
         wait_all_after<PS>(acc);
         constexpr int P1 = HS & 1, OFF1 = GROUPS_PER_TAP == 2 ? HS * 32 : 0;
         using std::integral_constant;
@@ -583,10 +644,12 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 // One thread per dword of the fragment layout [OC/32][tap][KS][lane][4 dwords]:
 // lane l of a fragment holds filter (l % 32) and channels (l / 32) * 32 .. +31 of the step,
 // eight channels per dword, low nibble first.  Channels >= IC and filters >= OC are FP4 zero.
+// With pair set, [tap] runs over pairs of taps and the 2*KS half-steps of a pair are the KS
+// 32-channel words of its first tap followed by those of its second (zero if there is none).
 __global__ __launch_bounds__(256)
 void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__ frag,
-        const Geometry g, const int ks_n, const int oc_subs) {
-    const int taps = g.kh * g.kw;
+        const Geometry g, const int ks_n, const int oc_subs, const int pair) {
+    const int taps = pair ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
     const size_t total = (size_t)oc_subs * taps * ks_n * 64 * 4;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
@@ -594,15 +657,21 @@ void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__
     const int lane = (int)((i >> 2) & 63);
     const size_t f = i >> 8; // fragment index
     const int ks = (int)(f % ks_n);
-    const int tap = (int)((f / ks_n) % taps);
+    int tap = (int)((f / ks_n) % taps);
     const int sub = (int)(f / ((size_t)ks_n * taps));
     const int oc = sub * 32 + (lane & 31);
-    const int c0 = ks * 64 + (lane >> 5) * 32 + dw * 8;
+    int c0 = ks * 64 + (lane >> 5) * 32 + dw * 8;
+    if (pair) {
+        const int word = 2 * ks + (lane >> 5); // of the 2*KS words of the pair
+        tap = 2 * tap + (word >= ks_n ? 1 : 0);
+        c0 = (word >= ks_n ? word - ks_n : word) * 32 + dw * 8;
+    }
+    const bool tap_exists = tap < g.kh * g.kw;
     const int kh = tap / g.kw, kw = tap % g.kw;
     uint32_t out = 0;
     for (int n = 0; n < 8; n++) {
         const int c = c0 + n;
-        if (oc < g.oc && c < g.ic) {
+        if (tap_exists && oc < g.oc && c < g.ic) {
             const size_t at = g.w_fmt == xnor_nn_weights_format_oihw
                 ? (((size_t)oc * g.ic + c) * g.kh + kh) * g.kw + kw
                 : (((size_t)kh * g.kw + kw) * g.ic + c) * g.oc + oc;
@@ -614,7 +683,16 @@ void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__
 
 // Steps per tap as the kernel is instantiated: ceil(IC/64), odd counts above 4 rounded up,
 // counts above 8 rounded up to 12 or 16 (the extra steps multiply FP4 zeros).
+// Pairing two taps per KS = ceil(IC/32) steps pays when the number of 32-channel words is odd
+// (otherwise every tap ends on a half-empty step) and small enough for the register file.
+bool pair_taps(const Geometry &g) {
+    const int taps = g.kh * g.kw;
+    if ((g.xw & 1) == 0 || g.xw > 5 || taps < 2) return false;
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_PAIR")) return e[0] == '1';
+    return ((taps + 1) / 2) * g.xw < taps * ((g.xw + 1) / 2);
+}
 int steps_per_tap(const Geometry &g) {
+    if (pair_taps(g)) return g.xw; // per pair of taps
     const int ks = (g.ic + 63) / 64;
     if (ks > 8) return (ks + 3) / 4 * 4; // 12 or 16
     return ks > 4 && (ks & 1) ? ks + 1 : ks;
@@ -641,7 +719,8 @@ int max_tile_rows(const Geometry &g, uint32_t mt) {
 
 size_t lds_bytes(const Geometry &g, int ps) {
     const size_t rows = (size_t)max_tile_rows(g, 32 * ps);
-    return TABLE_BYTES + ALPHA_BYTES + (1 + rows) * (steps_per_tap(g) * 32 + ROW_PAD)
+    const size_t row_bytes = pair_taps(g) ? g.xw * 16 : steps_per_tap(g) * 32 + ROW_PAD;
+    return TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
         + (rows + 1 + 32 * ps) * sizeof(float);
 }
 
@@ -656,7 +735,7 @@ int pick_ps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
         const int v = atoi(e);
         if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT
-                && !(v == 4 && steps_per_tap(g) > 8))
+                && !(v == 4 && (steps_per_tap(g) > 8 || (pair_taps(g) && g.xw >= 3))))
             return v;
     }
     const int chunks = (g.oc + NT - 1) / NT;
@@ -666,7 +745,8 @@ int pick_ps(const Geometry &g) {
     double best_cost = 0;
     for (int ps = 4; ps >= 1; ps--) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
-        if (ps == 4 && steps_per_tap(g) > 8) continue; // would not fit the register file
+        // would not fit the register file
+        if (ps == 4 && (steps_per_tap(g) > 8 || (pair_taps(g) && g.xw >= 3))) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
         const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
@@ -677,7 +757,7 @@ int pick_ps(const Geometry &g) {
     return best;
 }
 
-template <int KS, int PS>
+template <int KS, int PS, bool PAIR>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
@@ -689,25 +769,25 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const size_t lds = lds_bytes(g, PS);
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (popc)
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true>), grid, block, lds, s, xbits,
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR>), grid, block, lds, s, xbits,
                 wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
     else
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false>), grid, block, lds, s, xbits,
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR>), grid, block, lds, s, xbits,
                 wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
     return hipGetLastError();
 }
 
-template <int KS>
+template <int KS, bool PAIR = false>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
     switch (g.mfma_ps) {
-    case 1: return launch_mfma<KS, 1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma<KS, 2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma<KS, 3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 4: return launch_mfma<KS, 4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma<KS, 3, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 4: return launch_mfma<KS, 4, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }
@@ -729,26 +809,36 @@ int mfma_tile_blocks(const Geometry &g) {
 }
 
 size_t mfma_weight_bytes(const Geometry &g) {
-    return (size_t)oc_subblocks(g) * g.kh * g.kw * steps_per_tap(g) * 1024;
+    const int units = pair_taps(g) ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
+    return (size_t)oc_subblocks(g) * units * steps_per_tap(g) * 1024;
 }
 
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
         hipStream_t s) {
     const size_t dwords = mfma_weight_bytes(g) / 4;
     hipLaunchKernelGGL(pack_weights_fp4_kernel, dim3((unsigned)((dwords + 255) / 256)),
-            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g));
+            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g), pair_taps(g) ? 1 : 0);
     return hipGetLastError();
 }
 
 const char *mfma_kernel_name(const Geometry &g) {
     static thread_local char name[64];
-    snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d>", steps_per_tap(g), g.mfma_ps);
+    snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", steps_per_tap(g), g.mfma_ps,
+            pair_taps(g) ? ",PAIR" : "");
     return name;
 }
 
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
         float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s) {
+    if (pair_taps(g)) {
+        switch (g.xw) {
+        case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+        case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+        case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+        }
+        return hipErrorInvalidValue;
+    }
     switch (steps_per_tap(g)) {
     case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
