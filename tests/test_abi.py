@@ -96,8 +96,9 @@ def test_init_fills_descriptor_like_the_reference():
     assert c.state and all((c.binarize_weights, c.binarize_data, c.calculate_k, c.forward))
     assert c.resource_size[capi.RES_BIN_SRC] == 4 * 27 * 27 * 3 * 4
     # packed sign words [OC/16][taps][words][16], then the same signs as FP4 matrix-core
-    # fragments [OC/32][taps][ceil(IC/64)][64 lanes][16 bytes]
-    assert c.resource_size[capi.RES_BIN_WEIGHTS] == 16 * 25 * 3 * 16 * 4 + 8 * 25 * 2 * 64 * 16
+    # fragments [OC/32][units][steps][64 lanes][16 bytes]; IC = 96 is three 32-channel words,
+    # an odd number, so a unit is a pair of taps (13 for 25 taps) of 3 steps
+    assert c.resource_size[capi.RES_BIN_WEIGHTS] == 16 * 25 * 3 * 16 * 4 + 8 * 13 * 3 * 64 * 16
     assert c.resource_size[capi.RES_A] == c.resource_size[capi.RES_K] == 4 * 27 * 27 * 4
     assert c.resource_size[capi.RES_ALPHA] == 256 * 4
     assert c.resource_size[capi.RES_OPERATIONS_COUNT] == 27 * 27 * 4
