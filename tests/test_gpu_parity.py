@@ -250,6 +250,25 @@ def test_strided_shapes_on_the_matrix_core_kernel(oracle, t):
     run_and_compare(oracle, d, x, w)
 
 
+@pytest.mark.parametrize("t", [
+    (1, 512, 64, 112, 112, 3, 3, 1, 1, 1, 1),  # 258 staged pixels of 272 bytes
+    (1, 1024, 40, 56, 56, 3, 3, 1, 1, 1, 1),   # 16 steps per tap on a 56 x 56 image
+    (1, 256, 32, 60, 60, 7, 7, 2, 2, 3, 3),    # 7 x 7 stride 2: seven image rows and more
+    (1, 96, 70, 120, 120, 11, 11, 4, 4, 2, 2), # 11 x 11 stride 4, paired taps
+], ids=shapes.shape_id)
+def test_tiles_that_need_more_than_64_kb_of_lds(oracle, t):
+    """The matrix-core kernel keeps every input pixel a tile touches in LDS; a gfx950
+    workgroup may use up to 160 KB of it, which has to be asked for above 64 KB."""
+    d = shapes.as_dims(t)
+    x = synth.normal(81, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(82, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    conv_name = make(d, w).kernel_name(0)
+    assert conv_name.startswith("conv_mfma"), conv_name
+    run_and_compare(oracle, d, x, w)
+
+
 def _random_case(rng):
     kh, kw = int(rng.integers(1, 8)), int(rng.integers(1, 8))
     ph, pw = int(rng.integers(0, 4)), int(rng.integers(0, 4))

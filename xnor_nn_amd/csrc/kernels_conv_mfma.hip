@@ -45,7 +45,9 @@ constexpr int NT = 256;       // filters per workgroup (4 waves x 64)
 constexpr int ROW_PAD = 16;   // spare bytes per LDS row
 constexpr int TABLE_BYTES = 1024;
 constexpr int ALPHA_BYTES = NT * 4;
-constexpr int LDS_LIMIT = 64 * 1024;
+constexpr int LDS_LIMIT = 160 * 1024;    // a gfx950 workgroup may take the whole LDS of its CU
+constexpr int LDS_DEFAULT = 64 * 1024;   // above this the kernel has to ask for it
+constexpr int LDS_TWO_PER_CU = 80 * 1024;
 
 // First and last input pixel (flattened index) that the tile of mt output pixels starting
 // at tile*mt can touch with an in-bounds tap: from the start of the first input row of its
@@ -751,7 +753,10 @@ int pick_ps(const Geometry &g) {
         const double per_simd = tiles * chunks * waves_per_block / simds;
         const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
                                              : per_simd + 0.5;
-        const double cost = (busiest < 1 ? 1 : busiest) * (ps + 0.5);
+        // a tile that needs more than half the LDS runs alone on its CU: nothing covers its
+        // staging and its epilogue
+        const double alone = lds_bytes(g, ps) > (size_t)LDS_TWO_PER_CU ? 1.15 : 1.0;
+        const double cost = (busiest < 1 ? 1 : busiest) * (ps + 0.5) * alone;
         if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
     }
     return best;
@@ -768,6 +773,13 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const int rows = max_tile_rows(g, 32 * PS);
     const size_t lds = lds_bytes(g, PS);
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
+    if (lds > (size_t)LDS_DEFAULT) {
+        const void *fn = popc ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR>
+                              : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR>;
+        const hipError_t e = hipFuncSetAttribute(fn,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR>), grid, block, lds, s, xbits,
                 wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
@@ -795,7 +807,7 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 } // namespace
 
 // The matrix-core kernel covers convolutions with up to 1024 input channels whose
-// tile of input rows fits 64 KB of LDS; everything else runs the XNOR/popcount kernel.
+// tile of input rows fits the 160 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
 // Returns the tile size (32-pixel blocks per workgroup, 1..4) or 0 when not applicable.
 int mfma_tile_blocks(const Geometry &g) {
