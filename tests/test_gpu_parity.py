@@ -151,8 +151,9 @@ def test_tensor_formats(oracle, fmts, t):
     (2, 5, 3, 4, 6, 3, 3, 1, 1, 1, 1),        # oc below one filter group
     (1, 70, 20, 7, 5, 3, 3, 2, 2, 1, 1),      # stride 2, ic and oc ragged
     (3, 33, 17, 6, 6, 5, 5, 1, 1, 2, 2),      # one bit past a word
-    (1, 1100, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # more than 1024 channels
+    (1, 1100, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # more than 1024 channels: two parts of 12 steps
     (1, 3700, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # ic*kh*kw > 32767: int32 words upstream
+    (1, 4100, 16, 3, 3, 3, 3, 1, 1, 1, 1),    # more than 4096 channels: XNOR/popcount kernel
     (5, 64, 64, 5, 9, 1, 1, 1, 1, 0, 0),      # 1x1 filter
     (2, 16, 32, 8, 8, 3, 3, 1, 1, 0, 0),      # no padding
     (1, 24, 16, 12, 12, 7, 7, 3, 3, 3, 3),    # big filter, stride 3
@@ -267,6 +268,33 @@ def test_tiles_that_need_more_than_64_kb_of_lds(oracle, t):
     conv_name = make(d, w).kernel_name(0)
     assert conv_name.startswith("conv_mfma"), conv_name
     run_and_compare(oracle, d, x, w)
+
+
+@pytest.mark.parametrize("t,parts", [
+    ((2, 2048, 130, 7, 7, 1, 1, 1, 1, 0, 0), ("KS=16", "PARTS=2")),   # ResNet-50 style 1x1
+    ((1, 1536, 64, 9, 8, 3, 3, 1, 1, 1, 1), ("KS=12", "PARTS=2")),    # 24 steps, no padding
+    ((1, 2500, 40, 6, 6, 3, 3, 2, 2, 1, 1), ("KS=16", "PARTS=3")),    # 40 steps (run as 48), stride 2
+    ((1, 4096, 300, 4, 4, 2, 2, 1, 1, 0, 0), ("KS=16", "PARTS=4")),  # the most the kernel takes
+    ((3, 1100, 70, 12, 12, 3, 3, 1, 1, 1, 1), ("KS=12", "PARTS=2")),   # several tiles per image
+], ids=lambda v: shapes.shape_id(v) if len(v) == 11 else "-".join(v))
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+def test_more_than_1024_channels_on_the_matrix_core_kernel(oracle, t, parts, layout):
+    """Above 1024 input channels the kernel walks every tap once per part of 768 or 1024
+    channels; the fragments of a part follow those of the part before."""
+    d = shapes.as_dims(t)
+    x = synth.normal(91, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::6] = 0.0
+    w = synth.normal(92, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    fmts = (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW)
+    if layout == "nhwc":
+        fmts = (capi.FMT_NHWC, capi.FMT_HWIO, capi.FMT_NHWC)
+        x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+        w = np.ascontiguousarray(w.transpose(2, 3, 1, 0))
+    conv_name = make(d, w, fmts).kernel_name(0)
+    assert conv_name.startswith("conv_mfma") and all(p in conv_name for p in parts), conv_name
+    run_and_compare(oracle, d, x, w, fmts)
 
 
 def _random_case(rng):

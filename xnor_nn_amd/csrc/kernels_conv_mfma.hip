@@ -155,14 +155,17 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
 // KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4 and to 12 or 16
 // above 8), PS = 32-pixel
 // blocks per workgroup tile.
-template <int KS, int PS, bool RAW, bool PAIR>
+// DEEP (more than 1024 channels): the channels of a pixel are cut into ic_parts parts of
+// 64*KS, and every (tap, part) is walked like a tap of its own whose rows start
+// 32*KS bytes further into the same LDS rows.
+template <int KS, int PS, bool RAW, bool PAIR, bool DEEP>
 __global__ __launch_bounds__(256, 2)
 void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
         const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
         const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
         const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
-        float *__restrict__ k_out, const float inv_khw) {
+        float *__restrict__ k_out, const float inv_khw, const int ic_parts) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
@@ -170,7 +173,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // PAIR (an odd number KS of 32-channel words per pixel): two taps share KS steps, so no
     // step is half empty; the rows then hold exactly KS words (16*KS bytes is 4 mod 8 dwords,
     // which keeps the fragment reads conflict-free without padding).
-    constexpr int ROW_BYTES = PAIR ? KS * 16 : KS * 32 + ROW_PAD;
+    const int ROW_BYTES = DEEP ? ic_parts * KS * 32 + ROW_PAD
+                               : PAIR ? KS * 16 : KS * 32 + ROW_PAD;
     // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows)
     float *a_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES);
     float *k_lds = a_lds + max_rows + 1; // K of the tile's pixels, same case
@@ -195,7 +199,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
     const int chunk = unit - tile * oc_chunks;
     // "taps" below are the units the main loop walks over: kernel taps, or pairs of them
-    const int taps = PAIR ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
+    const int taps = PAIR ? (g.kh * g.kw + 1) / 2 : DEEP ? g.kh * g.kw * ic_parts : g.kh * g.kw;
 
     // ---- which input pixels does the tile touch ------------------------------------------
     const uint32_t p_first = tile * MT;
@@ -355,8 +359,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // LDS address of each pixel's row for tap (kh, kw): a fixed offset from the row of tap
     // (0,0), or the zero row when the tap falls outside the image.  Every in-bounds tap of a
     // tile lies inside the span of rows the tile has staged (tile_span).
+    int npart = 0; // DEEP: channel part of the tap that nkh, nkw (below) name
     auto tap_rows = [&](int kh, int kw, uint32_t (&out)[PS]) {
-        const uint32_t shift = (uint32_t)((kh * g.iw + kw) * ROW_BYTES);
+        const uint32_t shift = (uint32_t)((kh * g.iw + kw) * ROW_BYTES)
+            + (DEEP ? (uint32_t)(npart * KS * 32) : 0u);
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
             const uint32_t ok = (rowmask[ps] >> kh) & (colmask[ps] >> kw) & 1u;
@@ -366,8 +372,11 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     int nkh = 0, nkw = 0; // the tap after the one being multiplied (the last tap repeats)
     bool ntap_valid = true; // PAIR: false once the walk has run past the last tap
     auto advance_tap = [&]() {
-        if (nkw + 1 < g.kw) nkw++;
-        else if (nkh + 1 < g.kh) { nkw = 0; nkh++; }
+        if constexpr (DEEP) {
+            if (npart + 1 < ic_parts) { npart++; return; }
+        }
+        if (nkw + 1 < g.kw) { nkw++; npart = 0; }
+        else if (nkh + 1 < g.kh) { nkw = 0; nkh++; npart = 0; }
         else ntap_valid = false;
     };
     // PAIR: rows of the two taps of a pair (index 0 and 1); a missing second tap (odd number
@@ -648,10 +657,13 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 // eight channels per dword, low nibble first.  Channels >= IC and filters >= OC are FP4 zero.
 // With pair set, [tap] runs over pairs of taps and the 2*KS half-steps of a pair are the KS
 // 32-channel words of its first tap followed by those of its second (zero if there is none).
+// With ic_parts > 1, [tap] runs over (tap, channel part) with the part innermost, and part p
+// holds channels 64*KS*p onwards.
 __global__ __launch_bounds__(256)
 void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__ frag,
-        const Geometry g, const int ks_n, const int oc_subs, const int pair) {
-    const int taps = pair ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
+        const Geometry g, const int ks_n, const int oc_subs, const int pair,
+        const int ic_parts) {
+    const int taps = pair ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw * ic_parts;
     const size_t total = (size_t)oc_subs * taps * ks_n * 64 * 4;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
@@ -663,6 +675,10 @@ void pack_weights_fp4_kernel(const float *__restrict__ w, uint32_t *__restrict__
     const int sub = (int)(f / ((size_t)ks_n * taps));
     const int oc = sub * 32 + (lane & 31);
     int c0 = ks * 64 + (lane >> 5) * 32 + dw * 8;
+    if (ic_parts > 1) {
+        c0 += (tap % ic_parts) * ks_n * 64;
+        tap /= ic_parts;
+    }
     if (pair) {
         const int word = 2 * ks + (lane >> 5); // of the 2*KS words of the pair
         tap = 2 * tap + (word >= ks_n ? 1 : 0);
@@ -693,9 +709,33 @@ bool pair_taps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PAIR")) return e[0] == '1';
     return ((taps + 1) / 2) * g.xw < taps * ((g.xw + 1) / 2);
 }
+// More than 1024 channels: parts of 12 or 16 steps, as few padded steps as possible (the
+// fewer parts on a tie).  Sets the steps per part; returns the number of parts, 1 if the
+// channels fit one part.
+int channel_parts(const Geometry &g, int *steps = nullptr) {
+    const int ks = (g.ic + 63) / 64;
+    int best_parts = 1, best_steps = 16;
+    if (ks > 16) {
+        best_parts = 0;
+        for (int parts = 2; parts <= 6; parts++)
+            for (int steps = 12; steps <= 16; steps += 4)
+                if (parts * steps >= ks
+                        && (best_parts == 0 || parts * steps < best_parts * best_steps)) {
+                    best_parts = parts;
+                    best_steps = steps;
+                }
+    }
+    if (steps) *steps = best_steps;
+    return best_parts;
+}
 int steps_per_tap(const Geometry &g) {
     if (pair_taps(g)) return g.xw; // per pair of taps
     const int ks = (g.ic + 63) / 64;
+    if (ks > 16) {
+        int steps;
+        channel_parts(g, &steps);
+        return steps;
+    }
     if (ks > 8) return (ks + 3) / 4 * 4; // 12 or 16
     return ks > 4 && (ks & 1) ? ks + 1 : ks;
 }
@@ -721,7 +761,8 @@ int max_tile_rows(const Geometry &g, uint32_t mt) {
 
 size_t lds_bytes(const Geometry &g, int ps) {
     const size_t rows = (size_t)max_tile_rows(g, 32 * ps);
-    const size_t row_bytes = pair_taps(g) ? g.xw * 16 : steps_per_tap(g) * 32 + ROW_PAD;
+    const size_t row_bytes = pair_taps(g) ? g.xw * 16
+        : channel_parts(g) * steps_per_tap(g) * 32 + ROW_PAD;
     return TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
         + (rows + 1 + 32 * ps) * sizeof(float);
 }
@@ -762,7 +803,7 @@ int pick_ps(const Geometry &g) {
     return best;
 }
 
-template <int KS, int PS, bool PAIR>
+template <int KS, int PS, bool PAIR, bool DEEP = false>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
@@ -772,23 +813,36 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const dim3 grid(per_xcd * 8), block(256);
     const int rows = max_tile_rows(g, 32 * PS);
     const size_t lds = lds_bytes(g, PS);
+    const int parts = DEEP ? channel_parts(g) : 1;
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (lds > (size_t)LDS_DEFAULT) {
-        const void *fn = popc ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR>
-                              : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR>;
+        const void *fn = popc ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>
+                              : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>;
         const hipError_t e = hipFuncSetAttribute(fn,
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
     if (popc)
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
+                xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts);
     else
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR>), grid, block, lds, s, xbits,
-                wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw);
+        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>), grid, block, lds, s,
+                xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts);
     return hipGetLastError();
+}
+
+template <int KS>
+hipError_t launch_mfma_deep(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
+        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        const float *a_or_null, float *k_out, hipStream_t s) {
+    switch (g.mfma_ps) {
+    case 1: return launch_mfma<KS, 1, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma<KS, 2, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma<KS, 3, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    }
+    return hipErrorInvalidValue;
 }
 
 template <int KS, bool PAIR = false>
@@ -806,14 +860,14 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 
 } // namespace
 
-// The matrix-core kernel covers convolutions with up to 1024 input channels whose
+// The matrix-core kernel covers convolutions with up to 4096 input channels whose
 // tile of input rows fits the 160 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
 // Returns the tile size (32-pixel blocks per workgroup, 1..4) or 0 when not applicable.
 int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
         if (e[0] == 'v') return 0;
-    if ((g.ic + 63) / 64 > 16) return 0;
+    if ((g.ic + 63) / 64 > 64) return 0;
     if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
     if ((uint64_t)g.npix_out * g.oc * 4u >= 0xFFFFFFF0ull) return 0; // 32-bit output offsets
     if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
@@ -821,7 +875,7 @@ int mfma_tile_blocks(const Geometry &g) {
 }
 
 size_t mfma_weight_bytes(const Geometry &g) {
-    const int units = pair_taps(g) ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw;
+    const int units = pair_taps(g) ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw * channel_parts(g);
     return (size_t)oc_subblocks(g) * units * steps_per_tap(g) * 1024;
 }
 
@@ -829,14 +883,20 @@ hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *
         hipStream_t s) {
     const size_t dwords = mfma_weight_bytes(g) / 4;
     hipLaunchKernelGGL(pack_weights_fp4_kernel, dim3((unsigned)((dwords + 255) / 256)),
-            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g), pair_taps(g) ? 1 : 0);
+            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g), pair_taps(g) ? 1 : 0,
+            channel_parts(g));
     return hipGetLastError();
 }
 
 const char *mfma_kernel_name(const Geometry &g) {
-    static thread_local char name[64];
-    snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", steps_per_tap(g), g.mfma_ps,
-            pair_taps(g) ? ",PAIR" : "");
+    static thread_local char name[80];
+    const int parts = channel_parts(g);
+    if (parts > 1)
+        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d,PARTS=%d>",
+                steps_per_tap(g), g.mfma_ps, parts);
+    else
+        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", steps_per_tap(g),
+                g.mfma_ps, pair_taps(g) ? ",PAIR" : "");
     return name;
 }
 
@@ -850,6 +910,11 @@ hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
         }
         return hipErrorInvalidValue;
+    }
+    if (channel_parts(g) > 1) {
+        if (steps_per_tap(g) == 12)
+            return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+        return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
     switch (steps_per_tap(g)) {
     case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
