@@ -184,7 +184,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // otherwise.  The longer lead hides more of the L2 latency of the fragment stream
     // (conv4 MB 256: main loop 11.9 -> 10.9 us per wave).
     // Above 8 steps per tap (more than 512 channels) a group is a quarter of a tap.
-    constexpr int HS = PAIR ? KS : KS > 8 ? KS / 4
+    constexpr int HS = PAIR ? KS : (KS > 8 || (KS == 8 && PS == 4)) ? KS / 4
         : (KS % 2 == 0 && KS >= 4 && (PS > 3 || 40 * PS + 16 * KS > 216)) ? KS / 2 : KS;
     constexpr int GROUPS_PER_TAP = KS / HS; // 1, 2 or 4
 
