@@ -344,13 +344,22 @@ def test_random_shapes_strides_and_layouts(oracle, seed):
         done += 1
 
 
-def test_forward_pass_captured_in_a_hip_graph(oracle, gpu):
+@pytest.mark.parametrize("case", ["conv4", "tile_above_64_kb"])
+def test_forward_pass_captured_in_a_hip_graph(oracle, gpu, case):
     """The three executors enqueue kernels only (no allocation, no memset, no host
     synchronisation when the tensors are on the device), so a caller may capture them in a
     HIP graph.  Every replay, with eager passes and synchronisations in between, must give
-    the eager result bit for bit."""
+    the eager result bit for bit.  The second case is a tile that has to ask for more than
+    64 KB of LDS at every launch, captured ones included."""
     import torch
-    d, x, w = synth.make_workload("alexnet_conv4_mb256", 24)
+    if case == "conv4":
+        d, x, w = synth.make_workload("alexnet_conv4_mb256", 24)
+    else:
+        d = shapes.as_dims((2, 512, 64, 112, 112, 3, 3, 1, 1, 1, 1))
+        x = synth.normal(95, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+            d["mb"], d["ic"], d["ih"], d["iw"])
+        w = synth.normal(96, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+            d["oc"], d["ic"], d["kh"], d["kw"])
     x2 = np.ascontiguousarray(x[::-1])
     s = oracle_shape(oracle, d)
     want, want2 = oracle.forward(s, x, w)["dst"], oracle.forward(s, x2, w)["dst"]

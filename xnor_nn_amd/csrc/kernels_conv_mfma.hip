@@ -27,6 +27,7 @@
 //   * PS (1 to 4) is chosen per problem so that the waves divide evenly over the SIMDs:
 //     for 43264 pixels, PS = 3 gives 1.76 waves per SIMD (2 in the busiest), PS = 4 gives
 //     1.32 (also 2, but each a third longer).
+#include <atomic>
 #include <cstdlib>
 #include <type_traits>
 
@@ -48,6 +49,7 @@ constexpr int ALPHA_BYTES = NT * 4;
 constexpr int LDS_LIMIT = 160 * 1024;    // a gfx950 workgroup may take the whole LDS of its CU
 constexpr int LDS_DEFAULT = 64 * 1024;   // above this the kernel has to ask for it
 constexpr int LDS_TWO_PER_CU = 80 * 1024;
+constexpr int MAX_DEVICES = 64;
 
 // First and last input pixel (flattened index) that the tile of mt output pixels starting
 // at tile*mt can touch with an in-bounds tap: from the start of the first input row of its
@@ -816,11 +818,21 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const int parts = DEEP ? channel_parts(g) : 1;
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (lds > (size_t)LDS_DEFAULT) {
-        const void *fn = popc ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>
-                              : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>;
-        const hipError_t e = hipFuncSetAttribute(fn,
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
+        // asked for once per kernel, device and size (what has been granted is remembered)
+        static std::atomic<size_t> granted[2][MAX_DEVICES];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+            return hipErrorInvalidDevice;
+        std::atomic<size_t> &have = granted[popc ? 1 : 0][dev];
+        if (lds > have.load(std::memory_order_acquire)) {
+            const void *fn = popc
+                ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>
+                : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>;
+            const hipError_t e = hipFuncSetAttribute(fn,
+                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+            have.store(lds, std::memory_order_release);
+        }
     }
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
