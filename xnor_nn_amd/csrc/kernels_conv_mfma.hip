@@ -30,6 +30,7 @@
 #include <atomic>
 #include <cstdlib>
 #include <type_traits>
+#include <utility>
 
 #include "plan.hpp"
 
@@ -93,13 +94,36 @@ __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c)
 //     before it and ahead of those that follow, which are the ones that consume the
 //     awaited registers.  The awaited registers themselves are deliberately not operands
 //     of the wait: a read-write operand lets the compiler copy the register on the way in,
-//     and a copy of a register whose load is still in flight copies stale data.  For the
-//     same reason nothing is in flight when control passes a loop edge.
+//     and a copy of a register whose load is still in flight copies stale data.
 //   * fetch_rows_after first waits for the LDS reads of the previous call (the operands of
 //     the matrix instructions that follow it) and then starts the reads for the step after,
 //     which the 2*PS matrix instructions of the current step cover.
-__device__ __forceinline__ void load_frag_async(v4i &dst, const v4i *src) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src));
+//   * Weight fragments are asked for one group (HS steps) ahead, two per step, and awaited
+//     by count: vector memory returns in order, so "at most 2*HS loads outstanding" at step
+//     hs means the two fragments of step hs, asked for 2*HS loads ago, have arrived.
+//   * A register must stay named by the program for as long as a load into it is on the
+//     way: the compiler takes the load for an ordinary definition and hands a register it
+//     thinks dead to the next computation, which the late data then overwrites.  Inside
+//     the loops both fragment sets are live by construction; after them they are named once
+//     more behind the final wait.  tests/test_isa_hazards.py checks the machine code of
+//     every variant for this.
+template <int... I, class F>
+__device__ __forceinline__ void static_for_each(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) { // f(integral_constant<int, 0>) ... <N-1>
+    static_for_each(std::make_integer_sequence<int, N>{}, f);
+}
+
+// Fragment loads are buffer loads: the lane's byte offset is one VGPR that never changes, the
+// fragment is a scalar offset plus an immediate, so a load costs no vector instruction for
+// its address.
+template <int IMM>
+__device__ __forceinline__ void load_frag_async(v4i &dst, const v4i desc, const uint32_t voff,
+        const uint32_t soff) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
+            : "=v"(dst) : "v"(voff), "s"(desc), "s"(soff), "n"(IMM));
 }
 #define XNOR_ACC1 "+v"(acc[0][0]), "+v"(acc[1][0])
 #define XNOR_ACC2 "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1])
@@ -114,30 +138,30 @@ __device__ __forceinline__ void wait_all_after(v16f (&acc)[2][PS]) {
     else if constexpr (PS == 3) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC3);
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : XNOR_ACC4);
 }
-template <int PS>
+template <int PS, int VM>
 __device__ __forceinline__ void fetch_rows_after(v4i (&bn)[PS], const uint32_t (&a)[PS],
         v16f (&acc)[2][PS]) {
     if constexpr (PS == 1)
-        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]"
+        asm volatile("s_waitcnt vmcnt(%[vm]) lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]"
                 : [b0] "=&v"(bn[0]), XNOR_ACC1
-                : [a0] "v"(a[0]));
+                : [a0] "v"(a[0]), [vm] "n"(VM));
     else if constexpr (PS == 2)
-        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+        asm volatile("s_waitcnt vmcnt(%[vm]) lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
                      "ds_read_b128 %[b1], %[a1]"
                 : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), XNOR_ACC2
-                : [a0] "v"(a[0]), [a1] "v"(a[1]));
+                : [a0] "v"(a[0]), [a1] "v"(a[1]), [vm] "n"(VM));
     else if constexpr (PS == 3)
-        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+        asm volatile("s_waitcnt vmcnt(%[vm]) lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
                      "ds_read_b128 %[b1], %[a1]\n\tds_read_b128 %[b2], %[a2]"
                 : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), [b2] "=&v"(bn[2]), XNOR_ACC3
-                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]));
+                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [vm] "n"(VM));
     else
-        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
+        asm volatile("s_waitcnt vmcnt(%[vm]) lgkmcnt(0)\n\tds_read_b128 %[b0], %[a0]\n\t"
                      "ds_read_b128 %[b1], %[a1]\n\tds_read_b128 %[b2], %[a2]\n\t"
                      "ds_read_b128 %[b3], %[a3]"
                 : [b0] "=&v"(bn[0]), [b1] "=&v"(bn[1]), [b2] "=&v"(bn[2]), [b3] "=&v"(bn[3]),
                   XNOR_ACC4
-                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]));
+                : [a0] "v"(a[0]), [a1] "v"(a[1]), [a2] "v"(a[2]), [a3] "v"(a[3]), [vm] "n"(VM));
 }
 #undef XNOR_ACC1
 #undef XNOR_ACC2
@@ -167,7 +191,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
         const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
         const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
-        float *__restrict__ k_out, const float inv_khw, const int ic_parts) {
+        float *__restrict__ k_out, const float inv_khw, const int ic_parts,
+        const uint32_t wfrag_bytes) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
@@ -347,16 +372,21 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // Weight fragments: [32-filter block][tap][step][lane], two register sets of HS steps
     // used in turn (a "group" is HS steps of one tap).  Group n+1 is requested before group
     // n is multiplied and awaited after its 2*PS*HS matrix instructions.
-    const v4i *wsrc[2];
+    const uint64_t wfrag_at = reinterpret_cast<uint64_t>(wfrag);
+    const v4i wdesc = {(int)(uint32_t)wfrag_at, (int)(uint32_t)((wfrag_at >> 32) & 0xFFFFu),
+                       (int)wfrag_bytes, 0x00020000};
+    const uint32_t wvoff = (uint32_t)lane * 16u;
+    uint32_t wbase[2]; // byte offset of this wave's two 32-filter blocks
 #pragma unroll
     for (int os = 0; os < 2; os++)
-        wsrc[os] = wfrag + (size_t)(oc_sub0 + os) * taps * KS * 64 + lane;
-    auto request = [&](int group, v4i (&w)[HS][2]) { // group = tap * GROUPS_PER_TAP + part
+        wbase[os] = (uint32_t)(oc_sub0 + os) * (uint32_t)(taps * KS) * 1024u;
+    // the two fragments of step hs of a group (group = tap * GROUPS_PER_TAP + part)
+    auto request_step = [&](int group, auto step, v4i (&w)[HS][2]) {
+        constexpr int hs = decltype(step)::value;
 #pragma unroll
-        for (int hs = 0; hs < HS; hs++)
-#pragma unroll
-            for (int os = 0; os < 2; os++)
-                load_frag_async(w[hs][os], wsrc[os] + ((size_t)group * HS + hs) * 64);
+        for (int os = 0; os < 2; os++)
+            load_frag_async<(hs & 3) * 1024>(w[hs][os], wdesc, wvoff,
+                    wbase[os] + (uint32_t)(group * HS + (hs & ~3)) * 1024u);
     };
     // LDS address of each pixel's row for tap (kh, kw): a fixed offset from the row of tap
     // (0,0), or the zero row when the tap falls outside the image.  Every in-bounds tap of a
@@ -423,11 +453,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     v4i b0[PS], b1[PS];   // pixel fragments of the current and the following step, in turn
     // One group with the fragments in wc, while those of the next group arrive in wn.
     // P0: which of b0/b1 holds the group's first step; OFF / NOFF: byte offset within a row of
-    // this group's and of the next group's first step.  In the paired loop the group after
-    // the last one is the last one again: loaded, awaited and never used.  MORE = false (the
-    // single group after the loop) fetches nothing beyond the group: a load whose result is
-    // never read must not exist, because its destination registers would be given to
-    // something else while it is still in flight.
+    // this group's and of the next group's first step.  In the loops the group after the
+    // last one is the last one again: loaded, awaited after the loops and never multiplied.
+    // MORE = false (the single group after the paired loop) asks for nothing.
     auto run_group = [&](auto more, auto newtap, auto p0, auto off, auto noff, int n,
                          const v4i (&wc)[HS][2], v4i (&wn)[HS][2]) {
         constexpr bool MORE = decltype(more)::value, NEWTAP = decltype(newtap)::value;
@@ -435,8 +463,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                       NOFF = decltype(noff)::value;
         uint32_t nextaddr[PS];
         uint32_t nextpair[PAIR ? 2 : 1][PAIR ? PS : 1];
+        const int next_group = min(n + 1, last_group);
         if constexpr (MORE) {
-            request(min(n + 1, last_group), wn);
             if constexpr (PAIR) {
                 pair_rows(nextpair);
             } else if constexpr (NEWTAP) { // the next group starts the next tap
@@ -447,12 +475,17 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                 for (int ps = 0; ps < PS; ps++) nextaddr[ps] = rowaddr[ps];
             }
         }
-#pragma unroll
-        for (int hs = 0; hs < HS; hs++) {
-            if (hs + 1 < HS || MORE) {
+        // Step hs first asks for the two fragments of step hs of the next group, then waits
+        // until its own two have arrived: they were asked for one group ago, and the 2*HS
+        // loads started since (vector memory returns in order) may still be under way.
+        constexpr int VM = MORE ? 2 * HS : 0;
+        static_for<HS>([&](auto step) {
+            constexpr int hs = decltype(step)::value;
+            if constexpr (MORE) request_step(next_group, step, wn);
+            if constexpr (hs + 1 < HS || MORE) {
                 uint32_t a[PS];
                 if constexpr (PAIR) {
-                    if (hs + 1 < HS) pair_addr(hs + 1, pairaddr, a);
+                    if constexpr (hs + 1 < HS) pair_addr(hs + 1, pairaddr, a);
                     else pair_addr(0, nextpair, a);
                 } else {
 #pragma unroll
@@ -460,16 +493,15 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                         a[ps] = hs + 1 < HS ? rowaddr[ps] + OFF + (hs + 1) * 32
                                             : nextaddr[ps] + NOFF;
                 }
-                if (((P0 + hs) & 1) == 0) fetch_rows_after<PS>(b1, a, acc);
-                else fetch_rows_after<PS>(b0, a, acc);
+                if constexpr (((P0 + hs) & 1) == 0) fetch_rows_after<PS, VM>(b1, a, acc);
+                else fetch_rows_after<PS, VM>(b0, a, acc);
             } else {
                 wait_all_after<PS>(acc); // the last fragments of the kernel are in
             }
-            if (((P0 + hs) & 1) == 0) mma(wc[hs], b0);
+            if constexpr (((P0 + hs) & 1) == 0) mma(wc[hs], b0);
             else mma(wc[hs], b1);
-        }
+        });
         if constexpr (MORE) {
-            wait_all_after<PS>(acc); // wn and the first pixel fragments of the next group are in
             if constexpr (PAIR) {
 #pragma unroll
                 for (int ps = 0; ps < PS; ps++) {
@@ -485,7 +517,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 
     v4i wa[HS][2], wb[HS][2];
     if (wave_has_filters) {
-        request(0, wa);
+        static_for<HS>([&](auto step) { request_step(0, step, wa); });
         if constexpr (PAIR) {
             pair_rows(pairaddr);
         } else {
@@ -503,9 +535,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         if constexpr (PAIR) {
             uint32_t a0[PS];
             pair_addr(0, pairaddr, a0);
-            fetch_rows_after<PS>(b0, a0, acc);
+            fetch_rows_after<PS, 0>(b0, a0, acc);
         } else {
-            fetch_rows_after<PS>(b0, rowaddr, acc);
+            fetch_rows_after<PS, 0>(b0, rowaddr, acc);
         }
         wait_all_after<PS>(acc);
         constexpr int P1 = HS & 1, OFF1 = GROUPS_PER_TAP == 2 ? HS * 32 : 0;
@@ -536,6 +568,16 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         if (n <= last_group) // odd number of groups (only with one group per tap)
             run_group(std::false_type{}, std::false_type{}, integral_constant<int, 0>{},
                     integral_constant<int, 0>{}, integral_constant<int, 0>{}, n, wa, wb);
+        // The last group of the loops has asked for fragments that nothing multiplies.  They
+        // are awaited here, and both register sets are named as inputs after the wait: a
+        // register that is dead after the loop would otherwise be handed to the epilogue's
+        // address arithmetic while its load is still on the way.
+        wait_all_after<PS>(acc);
+        static_for<HS>([&](auto step) {
+            constexpr int hs = decltype(step)::value;
+            const v4i a0 = wa[hs][0], a1 = wa[hs][1], c0 = wb[hs][0], c1 = wb[hs][1];
+            asm volatile("" : : "v"(a0), "v"(a1), "v"(c0), "v"(c1));
+        });
     }
 
     // ---- epilogue: register i of a 32x32 block holds filter 8*(i/4) + 4*(lane/32) + i%4,
@@ -837,11 +879,13 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
                 xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts);
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
+                (uint32_t)mfma_weight_bytes(g));
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>), grid, block, lds, s,
                 xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
-                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts);
+                FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
+                (uint32_t)mfma_weight_bytes(g));
     return hipGetLastError();
 }
 
@@ -883,6 +927,7 @@ int mfma_tile_blocks(const Geometry &g) {
     if (g.kh > 32 || g.kw > 32) return 0; // taps inside the image are kept as 32-bit masks
     if ((uint64_t)g.npix_out * g.oc * 4u >= 0xFFFFFFF0ull) return 0; // 32-bit output offsets
     if ((uint64_t)g.npix_in * g.xw > 0x7FFFFFFFull) return 0;
+    if (mfma_weight_bytes(g) >= 0xFFFFFFF0ull) return 0; // 32-bit fragment offsets
     return pick_ps(g);
 }
 
