@@ -187,6 +187,17 @@ def test_matrix_core_tile_sizes(oracle, gpu, monkeypatch, ps):
     run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
     d, x, w = synth.make_workload("vgg_512_mb32", 1)
     run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+    # paired taps over three words, and 12 steps per tap
+    d, x, w = synth.make_workload("alexnet_conv2_mb128", 2)
+    assert make(d, w).kernel_name(0) == "conv_mfma_fp4_kernel<KS=3,PS=%s,PAIR>" % ps
+    run_and_compare(oracle, d, x, w, device_tensors=True, gpu=gpu)
+    d = shapes.as_dims((2, 768, 70, 14, 14, 3, 3, 1, 1, 1, 1))
+    x = synth.normal(75, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(76, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    assert make(d, w).kernel_name(0) == "conv_mfma_fp4_kernel<KS=12,PS=%s>" % ps
+    run_and_compare(oracle, d, x, w)
 
 
 @pytest.mark.parametrize("pair", ["0", "1"])

@@ -818,11 +818,18 @@ size_t lds_bytes(const Geometry &g, int ps) {
 // which streams fewer weight bytes.  (Measured on MI355X: conv4 MB 256 PS 2/3/4 = 29.1 /
 // 28.5 / 32.2 us, ResNet 3x3 MB 64 = 87.3 / 90.7 / 83.2, VGG 512 MB 32 = 42.6 / 46.1 / 39.3,
 // conv2 shape MB 128 = 54.1 / 51.3 / 49.7.)
+// Four pixel blocks do not fit the register file with 16 steps per tap or with tap pairing
+// over five words (those variants spill), and are not instantiated for channel parts.
+bool tile_fits_registers(const Geometry &g, int ps) {
+    if (ps < 4) return true;
+    if (channel_parts(g) > 1) return false;
+    return pair_taps(g) ? g.xw < 5 : steps_per_tap(g) < 16;
+}
+
 int pick_ps(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_MFMA_PS")) {
         const int v = atoi(e);
-        if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT
-                && !(v == 4 && (steps_per_tap(g) > 8 || (pair_taps(g) && g.xw >= 3))))
+        if (v >= 1 && v <= 4 && lds_bytes(g, v) <= (size_t)LDS_LIMIT && tile_fits_registers(g, v))
             return v;
     }
     const int chunks = (g.oc + NT - 1) / NT;
@@ -832,8 +839,7 @@ int pick_ps(const Geometry &g) {
     double best_cost = 0;
     for (int ps = 4; ps >= 1; ps--) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
-        // would not fit the register file
-        if (ps == 4 && (steps_per_tap(g) > 8 || (pair_taps(g) && g.xw >= 3))) continue;
+        if (!tile_fits_registers(g, ps)) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
         const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
