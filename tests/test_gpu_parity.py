@@ -308,6 +308,33 @@ def test_more_than_1024_channels_on_the_matrix_core_kernel(oracle, t, parts, lay
     run_and_compare(oracle, d, x, w, fmts)
 
 
+@pytest.mark.parametrize("by_lane", [False, True])
+@pytest.mark.parametrize("t", [
+    (3, 384, 64, 13, 13, 3, 3, 1, 1, 1, 1),    # twelve slices, one round; ragged last tile
+    (2, 512, 32, 9, 7, 3, 3, 1, 1, 1, 1),      # sixteen slices in two rounds of eight waves
+    (5, 100, 16, 6, 5, 1, 1, 1, 1, 0, 0),      # last slice holds 4 channels: 7 of 8 pieces empty
+    (1, 36, 16, 10, 10, 3, 3, 1, 1, 1, 1),     # one full slice and one piece
+    (1, 4, 8, 17, 3, 1, 1, 1, 1, 0, 0),        # a single piece, 51 pixels
+    (2, 800, 16, 5, 5, 3, 3, 1, 1, 1, 1),      # 25 slices in three rounds
+], ids=shapes.shape_id)
+def test_nhwc_input_kernels(oracle, monkeypatch, t, by_lane):
+    """Channels-last input: the tiled kernel (whole cache lines per load, turned around through
+    LDS) and the one-lane-per-pixel kernel it falls back to for very deep inputs."""
+    if by_lane:
+        monkeypatch.setenv("XNOR_NN_HIP_NHWC", "lane")
+    d = shapes.as_dims(t)
+    x = synth.normal(97, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ih"], d["iw"], d["ic"])
+    x.ravel()[::5] = 0.0
+    x.ravel()[1::7] = -0.0
+    w = synth.normal(98, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    fmts = (capi.FMT_NHWC, capi.FMT_OIHW, capi.FMT_NCHW)
+    name = make(d, w, fmts).kernel_name(2)
+    assert name == ("binarize_nhwc_kernel" if by_lane else "binarize_nhwc_tiled_kernel"), name
+    run_and_compare(oracle, d, x, w, fmts)
+
+
 def _random_case(rng):
     kh, kw = int(rng.integers(1, 8)), int(rng.integers(1, 8))
     ph, pw = int(rng.integers(0, 4)), int(rng.integers(0, 4))

@@ -15,6 +15,7 @@ namespace {
 
 constexpr int TILE = 64;       // pixels per workgroup = lanes per wave
 constexpr int MAX_WAVES = 12;  // waves per workgroup
+constexpr int TURN_ROW = 36;   // floats per pixel row of the NHWC turn-around buffer (32 + 4)
 
 __device__ __forceinline__ uint32_t fbits(float v) { return __float_as_uint(v); }
 
@@ -44,14 +45,22 @@ __device__ __forceinline__ uint32_t top_bits(int n) {
 // tiles [x * tiles_per_xcd, (x+1) * tiles_per_xcd): the cache lines that straddle two
 // neighbouring tiles (a channel plane is rarely a multiple of 128 bytes) are fetched into
 // one L2 instead of two.  Workgroup b takes local tile b / 8 of XCD b % 8.
-template <bool WRITE_BITS, bool WRITE_A>
-__global__ __launch_bounds__(TILE * 16)
-void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
-        float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
+//
+// NHWC input (channel count a multiple of 4) runs the same tile: the 32 values of a slice are
+// then 128 contiguous bytes of a pixel.  A wave fetches them eight lanes to a pixel, so that
+// every load instruction reads eight whole cache lines, and turns the block around through
+// LDS into the lane = pixel layout (one lane per pixel straight from memory, 64 partial
+// cache lines per instruction, took 19.7 us where this takes 13.5 us, the NCHW kernel 13.3).
+template <bool NHWC, bool WRITE_BITS, bool WRITE_A>
+__device__ __forceinline__
+void binarize_tile(const float *__restrict__ x, uint32_t *__restrict__ bits,
+        float *__restrict__ a, const Geometry &g, const float inv_ic, const int rounds,
         const uint32_t ntiles, const uint32_t tiles_per_xcd) {
     extern __shared__ uint32_t lds[];
     float *chain = reinterpret_cast<float *>(lds); // [TILE]
     uint32_t *stage = lds + TILE;                  // [TILE][xw]
+    // NHWC: [waves][32 pixels][TURN_ROW floats], 16-byte aligned
+    float *turn = reinterpret_cast<float *>(lds + ((TILE + TILE * g.xw + 3) & ~3));
 
     const int lane = threadIdx.x & (TILE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -71,6 +80,45 @@ void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bi
         const uint32_t hw = pc - img * g.ihw;
         const int c0 = (r * nw + wave) * 32; // wave-uniform
         if (c0 >= g.ic) return;
+        if constexpr (NHWC) {
+            // Load i of the wave reads the slice of pixels 8i .. 8i+7 of the tile: eight
+            // lanes per pixel, 16 bytes each, i.e. eight whole cache lines per instruction.
+            // The wave then turns the 64 x 128 bytes around through its own piece of LDS
+            // (32 pixels at a time, rows of 144 bytes so that neither side has bank
+            // conflicts) to end up with the lane = pixel layout of the rest of the kernel.
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const int piece = lane & 7;
+            const int c = c0 + 4 * piece; // IC is a multiple of 4: a piece is inside or outside
+            v4f v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t q = tile * TILE + 8 * i + (lane >> 3);
+                const uint32_t qc = q < g.npix_in ? q : g.npix_in - 1;
+                // a piece past the last channel gets an offset outside the buffer: reads +0
+                const uint32_t off = c < g.ic ? qc * (uint32_t)g.ic * 4u + (uint32_t)c * 4u
+                                              : 0xFFFFFFF0u;
+                v[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                        src, off, 0, 0));
+            }
+            float *mine = turn + wave * (32 * TURN_ROW);
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    *reinterpret_cast<v4f *>(mine + (8 * i + (lane >> 3)) * TURN_ROW + 4 * piece)
+                        = v[4 * half + i];
+                if ((lane >> 5) == half) {
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const v4f r = *reinterpret_cast<const v4f *>(
+                                mine + (lane & 31) * TURN_ROW + 4 * u);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) t[4 * u + e] = r[e];
+                    }
+                }
+            }
+            return;
+        }
         // Buffer loads: one VGPR holds the lane's byte offset for all 32 loads, the channel
         // plane is a scalar offset (no 64-bit address arithmetic per load, fewer VGPRs).
         const uint32_t lane_off = (img * (uint32_t)(g.ic * g.ihw) + hw) * 4u;
@@ -133,6 +181,24 @@ void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bi
     process(t, tile);
 }
 
+template <bool WRITE_BITS, bool WRITE_A>
+__global__ __launch_bounds__(TILE * 16)
+void binarize_nchw_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
+        float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
+        const uint32_t ntiles, const uint32_t tiles_per_xcd) {
+    binarize_tile<false, WRITE_BITS, WRITE_A>(x, bits, a, g, inv_ic, rounds, ntiles,
+            tiles_per_xcd);
+}
+
+template <bool WRITE_BITS, bool WRITE_A>
+__global__ __launch_bounds__(TILE * 16)
+void binarize_nhwc_tiled_kernel(const float *__restrict__ x, uint32_t *__restrict__ bits,
+        float *__restrict__ a, const Geometry g, const float inv_ic, const int rounds,
+        const uint32_t ntiles, const uint32_t tiles_per_xcd) {
+    binarize_tile<true, WRITE_BITS, WRITE_A>(x, bits, a, g, inv_ic, rounds, ntiles,
+            tiles_per_xcd);
+}
+
 // Any source layout, one lane per pixel, channels visited in order.  Used for NHWC input
 // (reference src/bcast_binarize_data.cpp:56-57, src/bcast_calculate_k.cpp:59-60).
 template <bool WRITE_BITS, bool WRITE_A>
@@ -166,7 +232,8 @@ void binarize_generic_kernel(const float *__restrict__ x, uint32_t *__restrict__
     if (WRITE_A) a[p] = acc;
 }
 
-// NHWC input with IC a multiple of 4: a lane is a pixel and walks over its channels, which
+// NHWC input with IC a multiple of 4 and too many channels for the tiled kernel's LDS: a lane
+// is a pixel and walks over its channels, which
 // are contiguous, in order, 32 at a time (one packed word): eight 16-byte buffer loads per
 // word, the loads of the next three words in flight while the current one is folded into
 // the sign word and the running mean|x| (reference src/bcast_binarize_data.cpp:56-57,
@@ -254,8 +321,8 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
     k[p] = acc;
 }
 
-template <bool WRITE_BITS, bool WRITE_A>
-void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
+template <bool NHWC, bool WRITE_BITS, bool WRITE_A>
+void launch_tiled(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
     // At most twelve waves per workgroup, the slices split evenly over the rounds: with more
     // waves the hand-over chain of one workgroup gets long and too few workgroups are
     // resident to cover it (512 input channels: 14.1 us with 16 waves, 10.4 us with 2 x 8;
@@ -271,9 +338,26 @@ void launch_nchw(const Geometry &g, const float *x, uint32_t *bits, float *a, hi
     const int nw = (need + rounds - 1) / rounds;
     const uint32_t ntiles = (g.npix_in + TILE - 1) / TILE;
     const uint32_t per_xcd = (ntiles + 7) / 8;
-    const size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
-    hipLaunchKernelGGL((binarize_nchw_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
-            dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+    size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
+    if (NHWC) lds = ((lds + 15) & ~(size_t)15) + sizeof(float) * nw * 32 * TURN_ROW;
+    if (NHWC)
+        hipLaunchKernelGGL((binarize_nhwc_tiled_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
+                dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+    else
+        hipLaunchKernelGGL((binarize_nchw_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
+                dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+}
+
+// NHWC input runs the tiled kernel unless its LDS (chain, packed words, turn-around rows) would
+// not fit 64 KB (more than about a thousand channels); XNOR_NN_HIP_NHWC=lane forces the
+// one-lane-per-pixel kernel (for measurements).
+bool nhwc_by_lane(const Geometry &g) {
+    const char *e = getenv("XNOR_NN_HIP_NHWC");
+    if (e && e[0] == 'l') return true;
+    const int rounds = (g.xw + MAX_WAVES - 1) / MAX_WAVES;
+    const int nw = (g.xw + rounds - 1) / rounds;
+    return sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw) + 16
+        + sizeof(float) * nw * 32 * TURN_ROW > 64 * 1024;
 }
 
 } // namespace
@@ -292,15 +376,19 @@ static bool vector_nhwc(const Geometry &g) {
 
 const char *binarize_kernel_name(const Geometry &g) {
     return tiled_nchw(g) ? "binarize_nchw_kernel"
-        : vector_nhwc(g) ? "binarize_nhwc_kernel" : "binarize_generic_kernel";
+        : !vector_nhwc(g) ? "binarize_generic_kernel"
+        : nhwc_by_lane(g) ? "binarize_nhwc_kernel" : "binarize_nhwc_tiled_kernel";
 }
 
 hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
         float *a_or_null, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
     if (tiled_nchw(g)) {
-        if (a_or_null) launch_nchw<true, true>(g, x, bits, a_or_null, s);
-        else launch_nchw<true, false>(g, x, bits, nullptr, s);
+        if (a_or_null) launch_tiled<false, true, true>(g, x, bits, a_or_null, s);
+        else launch_tiled<false, true, false>(g, x, bits, nullptr, s);
+    } else if (vector_nhwc(g) && !nhwc_by_lane(g)) {
+        if (a_or_null) launch_tiled<true, true, true>(g, x, bits, a_or_null, s);
+        else launch_tiled<true, true, false>(g, x, bits, nullptr, s);
     } else if (vector_nhwc(g)) {
         const unsigned blocks = (g.npix_in + 255) / 256;
         if (a_or_null)
@@ -324,7 +412,9 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
     if (tiled_nchw(g)) {
-        launch_nchw<false, true>(g, x, nullptr, a, s);
+        launch_tiled<false, false, true>(g, x, nullptr, a, s);
+    } else if (vector_nhwc(g) && !nhwc_by_lane(g)) {
+        launch_tiled<true, false, true>(g, x, nullptr, a, s);
     } else if (vector_nhwc(g)) {
         const unsigned blocks = (g.npix_in + 255) / 256;
         hipLaunchKernelGGL((binarize_nhwc_kernel<false, true>), dim3(blocks), dim3(256), 0, s,
