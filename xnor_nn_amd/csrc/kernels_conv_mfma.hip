@@ -47,6 +47,7 @@ constexpr int NT = 256;       // filters per workgroup (4 waves x 64)
 constexpr int ROW_PAD = 16;   // spare bytes per LDS row
 constexpr int TABLE_BYTES = 1024;
 constexpr int ALPHA_BYTES = NT * 4;
+constexpr int TURN_ROW = 36;  // floats per pixel row of the NHWC turn-around buffer (32 + 4)
 constexpr int LDS_LIMIT = 160 * 1024;    // a gfx950 workgroup may take the whole LDS of its CU
 constexpr int LDS_DEFAULT = 64 * 1024;   // above this the kernel has to ask for it
 constexpr int LDS_TWO_PER_CU = 80 * 1024;
@@ -205,6 +206,10 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows)
     float *a_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES);
     float *k_lds = a_lds + max_rows + 1; // K of the tile's pixels, same case
+    // NHWC output: per wave 32 pixel rows of TURN_ROW floats to turn a block around in
+    // (an offset from smem, not a rounded pointer: the compiler has to see an LDS address)
+    float *turn_lds = reinterpret_cast<float *>(smem + ((TABLE_BYTES + ALPHA_BYTES
+            + (1 + max_rows) * ROW_BYTES + (max_rows + 1 + 32 * PS) * 4 + 15) & ~15));
     constexpr int MT = 32 * PS;
     // Weight fragments are fetched in groups of HS steps, one group ahead: a whole tap where
     // the registers allow it (8 VGPRs per step on top of 32 per pixel block), half a tap
@@ -528,9 +533,16 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     __syncthreads(); // FP4 rows are in place
     float kv[PS]; // K of this wave's pixels
 #pragma unroll
-    for (int ps = 0; ps < PS; ps++)
-        kv[ps] = RAW ? 0.f : fuse_k ? k_lds[ps * 32 + (lane & 31)]
-                                    : kplane[live[ps] ? pix[ps] : 0];
+    for (int ps = 0; ps < PS; ps++) kv[ps] = 0.f;
+    if (!RAW) { // two branches: one select of an LDS and a global pointer would be a flat load
+        if (fuse_k) {
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) kv[ps] = k_lds[ps * 32 + (lane & 31)];
+        } else {
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) kv[ps] = kplane[live[ps] ? pix[ps] : 0];
+        }
+    }
     if (wave_has_filters) {
         if constexpr (PAIR) {
             uint32_t a0[PS];
@@ -628,28 +640,6 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                 // alphas of the four filters 8*i4 + 4*lane_hi + 0..3 of this 32-filter block
                 const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
                 const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
-                if constexpr (!NCHW && !CHECK) {
-                    // NHWC: registers 4*i4 .. +3 are four consecutive filters of the lane's
-                    // pixel, i.e. 16 contiguous bytes; the two lane halves write 32 and
-                    // the wave's eight stores per pixel block fill 256 bytes of each pixel.
-                    if (vec4_ok) {
-                        const uint32_t soff = (uint32_t)(chunk * NT + (wave * 2 + os) * 32
-                                + 8 * i4) * 4u;
-#pragma unroll
-                        for (int ps = 0; ps < PS; ps++) {
-                            v4i q;
-#pragma unroll
-                            for (int ii = 0; ii < 4; ii++) {
-                                const float d = acc[os][ps][4 * i4 + ii];
-                                q[ii] = RAW ? (((int)d + n[ps]) / 2)
-                                            : (int)__float_as_uint(__fmul_rn(
-                                                      __fmul_rn(d, al[ii]), kv[ps]));
-                            }
-                            __builtin_amdgcn_raw_buffer_store_b128(q, outbuf, off1[ps], soff, 0);
-                        }
-                        continue;
-                    }
-                }
 #pragma unroll
                 for (int ii = 0; ii < 4; ii++) {
                     const int i = 4 * i4 + ii;
@@ -686,7 +676,54 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             }
         }
     };
+    // NHWC with whole cache lines: a 32-filter x 32-pixel block is scaled in the accumulator
+    // layout (a lane holds 4 x 4 consecutive filters of one pixel), written to the wave's own
+    // LDS rows and read back eight lanes to a pixel, so that a store instruction writes the
+    // 128 contiguous bytes of 8 pixels instead of 32 bytes of 32 pixels.  Rows of 144 bytes
+    // keep both sides free of bank conflicts.  A piece past OC (OC is a multiple of 4 here)
+    // or a pixel past the end gets an offset outside the buffer.
+    auto store_lines_nhwc = [&]() {
+        float *mine = turn_lds + wave * (32 * TURN_ROW);
+        const int piece = lane & 7, prow = lane >> 3;
+        const uint32_t left = g.npix_out - p_first; // pixels of the tile that exist
+#pragma unroll
+        for (int os = 0; os < 2; os++) {
+            const uint32_t fpiece = (uint32_t)(chunk * NT + (wave * 2 + os) * 32 + 4 * piece);
+            const uint32_t base = fpiece < (uint32_t)g.oc
+                ? ((p_first + (uint32_t)prow) * (uint32_t)g.oc + fpiece) * 4u : DROP;
+#pragma unroll
+            for (int ps = 0; ps < PS; ps++) {
+#pragma unroll
+                for (int i4 = 0; i4 < 4; i4++) {
+                    const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
+                    const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
+                    v4i q;
+#pragma unroll
+                    for (int ii = 0; ii < 4; ii++)
+                        q[ii] = (int)__float_as_uint(
+                                __fmul_rn(__fmul_rn(acc[os][ps][4 * i4 + ii], al[ii]), kv[ps]));
+                    *reinterpret_cast<v4i *>(mine + (lane & 31) * TURN_ROW + 8 * i4 + 4 * lane_hi)
+                        = q;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4i r = *reinterpret_cast<const v4i *>(
+                            mine + (8 * j + prow) * TURN_ROW + 4 * piece);
+                    const uint32_t in_tile = (uint32_t)(ps * 32 + 8 * j); // + prow
+                    const uint32_t voff = in_tile + (uint32_t)prow < left ? base : DROP;
+                    __builtin_amdgcn_raw_buffer_store_b128(r, outbuf, voff,
+                            in_tile * (uint32_t)g.oc * 4u, 0);
+                }
+            }
+        }
+    };
     const bool all_filters = chunk * NT + (wave + 1) * 64 <= g.oc; // wave-uniform
+    if constexpr (!RAW) {
+        if (vec4_ok) {
+            store_lines_nhwc();
+            return;
+        }
+    }
     if (nchw) {
         if (all_filters) store_tile(std::false_type{}, std::true_type{});
         else store_tile(std::true_type{}, std::true_type{});
@@ -807,17 +844,20 @@ size_t lds_bytes(const Geometry &g, int ps) {
     const size_t rows = (size_t)max_tile_rows(g, 32 * ps);
     const size_t row_bytes = pair_taps(g) ? g.xw * 16
         : channel_parts(g) * steps_per_tap(g) * 32 + ROW_PAD;
-    return TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
+    size_t bytes = TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
         + (rows + 1 + 32 * ps) * sizeof(float);
+    if (g.dst_fmt == xnor_nn_data_format_nhwc && (g.oc & 3) == 0) // turn-around rows, 4 waves
+        bytes = ((bytes + 15) & ~(size_t)15) + 4 * 32 * TURN_ROW * sizeof(float);
+    return bytes;
 }
 
 // 32-pixel blocks per tile.  Cost of a choice = (waves the busiest SIMD runs one after the
 // other) x (work per wave, plus half a block for the staging and epilogue every tile pays).
 // With few waves per SIMD the busiest one sets the pace, so the count is rounded up; with
 // many, the hardware's dynamic scheduling evens the load out.  Ties go to the larger tile,
-// which streams fewer weight bytes.  (Measured on MI355X: conv4 MB 256 PS 2/3/4 = 29.1 /
-// 28.5 / 32.2 us, ResNet 3x3 MB 64 = 87.3 / 90.7 / 83.2, VGG 512 MB 32 = 42.6 / 46.1 / 39.3,
-// conv2 shape MB 128 = 54.1 / 51.3 / 49.7.)
+// which streams fewer weight bytes.  (Measured on MI355X, PS 1/2/3/4: conv4 MB 256 = 34.7 /
+// 27.0 / 26.6 / 27.5 us, ResNet 3x3 MB 64 = 113 / 97.0 / 96.6 / 96.9, VGG 512 MB 32 = 49.2 /
+// 37.6 / 39.6 / 35.2, conv2 shape MB 128 = 58.2 / 46.3 / 45.5 / 44.3.)
 // Four pixel blocks do not fit the register file with 16 steps per tap or with tap pairing
 // over five words (those variants spill), and are not instantiated for channel parts.
 bool tile_fits_registers(const Geometry &g, int ps) {
@@ -847,7 +887,9 @@ int pick_ps(const Geometry &g) {
         // a tile that needs more than half the LDS runs alone on its CU: nothing covers its
         // staging and its epilogue
         const double alone = lds_bytes(g, ps) > (size_t)LDS_TWO_PER_CU ? 1.15 : 1.0;
-        const double cost = (busiest < 1 ? 1 : busiest) * (ps + 0.5) * alone;
+        // below two blocks the weight stream (2 KB per wave and step whatever the tile) sets
+        // the pace of a step, not the matrix instructions
+        const double cost = (busiest < 1 ? 1 : busiest) * ((ps < 2 ? 2 : ps) + 0.5) * alone;
         if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
     }
     return best;
