@@ -482,6 +482,23 @@ def test_upstream_example_programs_run_unchanged(gpu, exe):
         assert out.stdout.strip() == "success"
 
 
+@pytest.mark.parametrize("exe", ["test_only_convolution", "test_simple_net"])
+def test_upstream_performance_programs_run_unchanged(gpu, exe):
+    """The reference's performance programs (reference test/perf/test_only_convolution.cpp:
+    8192 forward calls with only user_dst set; test/perf/test_simple_net.cpp: every stage of
+    seven layer shapes on host buffers, AlexNet conv1 with stride 4 among them), compiled
+    unchanged and linked to this library by `make -C oracle examples`.  Both end by printing
+    the status string of their last call."""
+    import subprocess
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "oracle", "_ref", "examples", exe)
+    if not os.path.exists(path):
+        pytest.skip("performance programs not built (upstream sources were not mounted)")
+    out = subprocess.run([path], capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, (out.stdout[-2000:], out.stderr[-2000:])
+    assert out.stdout.strip().endswith("success"), out.stdout[-500:]
+
+
 def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
     """With the matrix-core kernel, calculate_k leaves the box filter to the convolution.
     The K plane must still be what calculate_k saw: (1) read back before any forward, (2)
