@@ -109,6 +109,8 @@ def main():
     ap.add_argument("--mb", type=int, default=None,
                     help="override the batch size of the workload (experiments only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-host", action="store_true",
+                    help="skip the three forward passes through host buffers")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="after the timed region, run one plain device-to-device copy of "
                          "this many MiB (a kernel of known traffic to scale rocprofv3's "
@@ -200,6 +202,28 @@ def main():
     torch.cuda.synchronize()
     stage_ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i in range(3)]
     gpu_ms = sum(e[0].elapsed_time(e[3]) for e in evs) / args.steps
+
+    # Spread of the step time: one event between consecutive steps.
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    torch.cuda.synchronize()
+    marks[0].record(stream)
+    for i in range(args.steps):
+        step()
+        marks[i + 1].record(stream)
+    torch.cuda.synchronize()
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+
+    # The same forward pass through host buffers (pageable numpy arrays, the way the
+    # reference's own callers use the API): PCIe copies included, never the headline.
+    host_ms = None
+    if not args.no_host:
+        import numpy as np
+        yh = np.empty((d["mb"], d["oc"], wf["oh"], wf["ow"]), np.float32)
+        conv.forward(x, yh)
+        t2 = time.perf_counter()
+        for _ in range(3):
+            conv.forward(x, yh)
+        host_ms = 1e3 * (time.perf_counter() - t2) / 3
     conv_s = conv_ms * 1e-3
     # Roofline of the convolution kernel.  The matrix-core kernel multiplies +-1 values as
     # FP4 operands, so its ceiling is the chip's dense FP4 MFMA rate.  The XNOR/popcount
@@ -230,9 +254,14 @@ def main():
         "timing": "ms_per_step: wall clock over the K steps; kernel_us (used by the rooflines): "
                   "one pair of HIP events over those K steps and one over K back-to-back "
                   "launches of the binarize kernel, convolution = difference; stage_ms: a "
-                  "further pass with events around every stage, event cost included",
+                  "further pass with events around every stage, event cost included; "
+                  "step_ms_between_events: one event between consecutive steps; "
+                  "host_buffers_ms_per_forward: three passes through pageable host arrays",
         "kernel_us": {"step": step_ms_events * 1e3, "binarize": bin_ms * 1e3,
                       "convolution": conv_ms * 1e3},
+        "step_ms_between_events": {"min": per_step[0], "median": per_step[len(per_step) // 2],
+                                   "max": per_step[-1]},
+        "host_buffers_ms_per_forward": host_ms,
         "gpu_ms_per_forward_with_events": gpu_ms,
         "stage_ms": {"binarize_data": stage_ms[0], "calculate_k": stage_ms[1],
                      "forward": stage_ms[2]},
