@@ -329,11 +329,10 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
         else
             (void)hipGetLastError();
     }
-    g.mfma_ps = mfma_tile_blocks(g);
-    g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
+    mfma_plan(g);
     g.wfrag_offset = (bit_bytes + 255) / 256 * 256;
     c->resource_size[xnor_nn_resource_bin_weights] =
-        g.use_mfma ? g.wfrag_offset + mfma_weight_bytes(g) : bit_bytes;
+        g.use_mfma ? g.wfrag_offset + g.mfma_wbytes : bit_bytes;
     c->resource_size[xnor_nn_resource_a] = (size_t)g.npix_in * 4;
     c->resource_size[xnor_nn_resource_k] = (size_t)g.npix_out * 4;
     c->resource_size[xnor_nn_resource_alpha] = (size_t)oc * 4;

@@ -903,9 +903,9 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
     const uint32_t units = tiles * chunks, per_xcd = (units + 7) / 8;
     const dim3 grid(per_xcd * 8), block(256);
-    const int rows = max_tile_rows(g, 32 * PS);
-    const size_t lds = lds_bytes(g, PS);
-    const int parts = DEEP ? channel_parts(g) : 1;
+    const int rows = g.mfma_rows;
+    const size_t lds = g.mfma_lds;
+    const int parts = g.mfma_parts;
     const v4i *wf = reinterpret_cast<const v4i *>(wfrag);
     if (lds > (size_t)LDS_DEFAULT) {
         // asked for once per kernel, device and size (what has been granted is remembered)
@@ -928,12 +928,12 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
                 xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
-                (uint32_t)mfma_weight_bytes(g));
+                g.mfma_wbytes);
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>), grid, block, lds, s,
                 xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
-                (uint32_t)mfma_weight_bytes(g));
+                g.mfma_wbytes);
     return hipGetLastError();
 }
 
@@ -968,7 +968,7 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
 // tile of input rows fits the 160 KB of LDS; everything else runs the XNOR/popcount kernel.
 // XNOR_NN_HIP_CONV=valu forces the latter (used to profile the two side by side).
 // Returns the tile size (32-pixel blocks per workgroup, 1..4) or 0 when not applicable.
-int mfma_tile_blocks(const Geometry &g) {
+static int mfma_tile_blocks(const Geometry &g) {
     if (const char *e = getenv("XNOR_NN_HIP_CONV"))
         if (e[0] == 'v') return 0;
     if ((g.ic + 63) / 64 > 64) return 0;
@@ -984,31 +984,44 @@ size_t mfma_weight_bytes(const Geometry &g) {
     return (size_t)oc_subblocks(g) * units * steps_per_tap(g) * 1024;
 }
 
+void mfma_plan(Geometry &g) {
+    g.mfma_ps = mfma_tile_blocks(g);
+    g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
+    g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
+    g.mfma_parts = 1;
+    g.mfma_lds = g.mfma_wbytes = 0;
+    if (!g.use_mfma) return;
+    g.mfma_steps = steps_per_tap(g);
+    g.mfma_pair = pair_taps(g) ? 1 : 0;
+    g.mfma_parts = channel_parts(g);
+    g.mfma_rows = max_tile_rows(g, 32 * g.mfma_ps);
+    g.mfma_lds = (uint32_t)lds_bytes(g, g.mfma_ps);
+    g.mfma_wbytes = (uint32_t)mfma_weight_bytes(g);
+}
+
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
         hipStream_t s) {
-    const size_t dwords = mfma_weight_bytes(g) / 4;
+    const size_t dwords = g.mfma_wbytes / 4;
     hipLaunchKernelGGL(pack_weights_fp4_kernel, dim3((unsigned)((dwords + 255) / 256)),
-            dim3(256), 0, s, w, frag, g, steps_per_tap(g), oc_subblocks(g), pair_taps(g) ? 1 : 0,
-            channel_parts(g));
+            dim3(256), 0, s, w, frag, g, g.mfma_steps, oc_subblocks(g), g.mfma_pair, g.mfma_parts);
     return hipGetLastError();
 }
 
 const char *mfma_kernel_name(const Geometry &g) {
     static thread_local char name[80];
-    const int parts = channel_parts(g);
-    if (parts > 1)
+    if (g.mfma_parts > 1)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d,PARTS=%d>",
-                steps_per_tap(g), g.mfma_ps, parts);
+                g.mfma_steps, g.mfma_ps, g.mfma_parts);
     else
-        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", steps_per_tap(g),
-                g.mfma_ps, pair_taps(g) ? ",PAIR" : "");
+        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", g.mfma_steps,
+                g.mfma_ps, g.mfma_pair ? ",PAIR" : "");
     return name;
 }
 
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
         float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s) {
-    if (pair_taps(g)) {
+    if (g.mfma_pair) {
         switch (g.xw) {
         case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
         case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
@@ -1016,12 +1029,12 @@ hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         }
         return hipErrorInvalidValue;
     }
-    if (channel_parts(g) > 1) {
-        if (steps_per_tap(g) == 12)
+    if (g.mfma_parts > 1) {
+        if (g.mfma_steps == 12)
             return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
         return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     }
-    switch (steps_per_tap(g)) {
+    switch (g.mfma_steps) {
     case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
     case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);

@@ -60,6 +60,11 @@ struct Geometry {
     int use_mfma;               // 1: stage 3 runs the FP4 matrix-core kernel
     int mfma_ps;                // its tile size in 32-pixel blocks (1..4)
     size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
+    // the matrix-core kernel's variant and sizes, fixed once by mfma_plan: steps per tap (or
+    // per pair of taps), tap pairing, channel parts, input pixels a tile stages at most, LDS
+    // bytes per workgroup, bytes of the weight fragments
+    int mfma_steps, mfma_pair, mfma_parts, mfma_rows;
+    uint32_t mfma_lds, mfma_wbytes;
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
 
@@ -98,7 +103,9 @@ hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         float *dst, int32_t *popc_or_null, hipStream_t s);
 hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
         hipStream_t s);
-int mfma_tile_blocks(const Geometry &g);
+// Decides whether the matrix-core kernel takes the problem and fills use_mfma, mfma_ps and
+// the mfma_* fields (everything the launch needs, so that a forward call computes nothing).
+void mfma_plan(Geometry &g);
 const char *mfma_kernel_name(const Geometry &g);
 size_t mfma_weight_bytes(const Geometry &g);
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
