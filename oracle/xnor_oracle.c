@@ -23,6 +23,12 @@
  *                        known-answer forward (reference
  *                        test/gtest/test_convolution_reference_forward.cpp:58-73);
  *                        brute-force +-1 dot products from the raw floats.
+ *   xo_binarize_weights_float
+ *                        bit-for-bit against oracle/_ref run on ONE OpenMP thread (the
+ *                        reference adds into a shared variable from a parallel loop without
+ *                        a reduction, reference src/binarize_weights_float.cpp:17-19, so
+ *                        only its one-thread result is defined); closed forms (all ones,
+ *                        alternating signs, -0.0 counts as >= 0); float64 mean.
  * No function is "parity unpinned".
  *
  * Floating point: every product and every sum is rounded to float separately and in the
@@ -264,4 +270,18 @@ void xo_convolution(const xo_shape_t *s, int oci_n,
             dst[di] = v;
         }
     }
+}
+
+/* Float "binarized" weights for a framework's backward pass
+ * (reference src/binarize_weights_float.cpp:3-25), in the order one thread runs it:
+ *   alpha = fl(sum over i in index order of from[i]) -- the weights themselves, not |w| --
+ *   alpha = fl(alpha * cckhw), cckhw = 1.f / elems;
+ *   to[i] = fl((from[i] >= 0.f ? 1.f : -1.f) * alpha)   (-0.0f compares >= 0). */
+void xo_binarize_weights_float(const xo_shape_t *s, const float *from, float *to) {
+    const int elems = s->oc * s->ic * s->kh * s->kw;
+    const float cckhw = 1.f / elems;
+    float alpha = 0.f;
+    for (int i = 0; i < elems; i++) alpha += from[i];
+    alpha *= cckhw;
+    for (int i = 0; i < elems; i++) to[i] = (from[i] >= .0f ? 1.f : -1.f) * alpha;
 }

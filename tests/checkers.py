@@ -48,6 +48,7 @@ class Oracle:
         lib.xo_calculate_k.argtypes = [P, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.xo_binarize_weights.argtypes = [P, C.c_int] + [C.c_void_p] * 4
         lib.xo_convolution.argtypes = [P, C.c_int] + [C.c_void_p] * 7
+        lib.xo_binarize_weights_float.argtypes = [P, C.c_void_p, C.c_void_p]
         self.lib = lib
 
     def shape(self, mb, oc, ic, ih, iw, kh, kw, sh, sw, ph, pw,
@@ -95,6 +96,12 @@ class Oracle:
                                 _fptr(k), _fptr(opc), _fptr(popc), _fptr(dst))
         return popc, dst
 
+    def binarize_weights_float(self, s, w):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        out = np.empty(w.shape, dtype=np.float32)
+        self.lib.xo_binarize_weights_float(C.byref(s), _fptr(w), _fptr(out))
+        return out
+
     def forward(self, s, x, w, oci=None):
         """Whole pipeline; returns a dict with every intermediate."""
         bsrc = self.binarize_data(s, x)
@@ -121,6 +128,28 @@ class RefLib:
     def __init__(self):
         os.environ["XNOR_NN_ISA"] = "2"
         self.lib = capi.bind(C.CDLL(REF_SO), capi.CORE_SYMBOLS)
+
+    def binarize_weights_float(self, dims, w, threads=1):
+        """xnor_nn_binarize_weights_float on `threads` OpenMP threads.  Only one thread gives
+        a defined result: the loop adds into a shared variable without a reduction
+        (reference src/binarize_weights_float.cpp:17-19)."""
+        lib = self.lib
+        omp = C.CDLL("libgomp.so.1")
+        c = capi.ConvolutionDesc()
+        assert lib.xnor_nn_init_convolution(
+            C.byref(c), capi.ALGORITHM_BCAST, capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW,
+            dims["mb"], dims["oc"], dims["ic"], dims["ih"], dims["iw"],
+            dims["kh"], dims["kw"], dims["sh"], dims["sw"], dims["ph"], dims["pw"]) == 0
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        out = np.empty(w.shape, dtype=np.float32)
+        before = omp.omp_get_max_threads()
+        omp.omp_set_num_threads(threads)
+        try:
+            lib.xnor_nn_binarize_weights_float(C.byref(c), w.ctypes.data, out.ctypes.data)
+        finally:
+            omp.omp_set_num_threads(before)
+        lib.xnor_nn_destroy_convolution(C.byref(c))
+        return out
 
     def forward(self, dims, x, w, algorithm=capi.ALGORITHM_BCAST,
                 fmts=(capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW), reps=1, timer=None):

@@ -499,6 +499,73 @@ def test_upstream_performance_programs_run_unchanged(gpu, exe):
     assert out.stdout.strip().endswith("success"), out.stdout[-500:]
 
 
+def test_binarize_weights_float(oracle, gpu):
+    """xnor_nn_binarize_weights_float on host and on device buffers: the signs follow
+    w >= 0 exactly (a negative zero counts as positive), every magnitude is the same float,
+    and that float is the mean of the weights.  The reference's own sum is only defined on one
+    thread (a data race otherwise, reference src/binarize_weights_float.cpp:17-19) and is
+    sequential there; the device sums 256 slices, so the mean is compared to 1e-6 of the mean
+    magnitude instead of bit for bit."""
+    import torch
+    d, _, w = synth.make_workload("alexnet_conv4_mb256", 1)
+    w = w.copy()
+    w.ravel()[::97] = -0.0
+    want = oracle.binarize_weights_float(oracle_shape(oracle, d), w)
+    conv = make(d, w)
+    host = np.empty_like(w)
+    conv.binarizeWeightsFloat(w, host)
+    dev = torch.empty(w.shape, dtype=torch.float32, device=gpu)
+    conv.binarizeWeightsFloat(torch.from_numpy(w).to(gpu), dev)
+    conv.close()
+    scale = float(np.mean(np.abs(w.astype(np.float64))))
+    for got in (host, dev.cpu().numpy()):
+        assert np.array_equal(np.signbit(got), np.signbit(want))
+        m = got[w >= 0][0]
+        assert np.all(got[w >= 0] == m) and np.all(got[w < 0] == -m)
+        assert abs(float(m) - float(want[w >= 0][0])) <= 1e-6 * scale
+        assert abs(float(m) - float(np.mean(w.astype(np.float64)))) <= 1e-6 * scale
+
+
+def test_pytorch_layer(oracle, gpu):
+    """xnor_nn_amd.torch_layer.XnorConv2d, the forward pass of the reference's Caffe layer for
+    PyTorch tensors: bit-identical to the oracle, rebuilt for a new batch size, new weights
+    only after weights_changed()."""
+    import torch
+    from xnor_nn_amd.torch_layer import XnorConv2d
+    d, x, w = synth.make_workload("alexnet_conv4_mb256", 3)
+    s = oracle_shape(oracle, d)
+    layer = XnorConv2d(d["ic"], d["oc"], (d["kh"], d["kw"]), stride=(d["sh"], d["sw"]),
+                       padding=(d["ph"], d["pw"]), weight=torch.from_numpy(w)).to(gpu)
+    xt = torch.from_numpy(x).to(gpu)
+    y = layer(xt)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32),
+                          oracle.forward(s, x, w)["dst"].view(np.uint32))
+    # another batch size builds another descriptor
+    d2 = dict(d, mb=2)
+    y2 = layer(xt[:2])
+    assert np.array_equal(y2.cpu().numpy().view(np.uint32),
+                          oracle.forward(oracle_shape(oracle, d2), x[:2], w)["dst"].view(np.uint32))
+    # new weights take effect once the layer is told
+    w2 = np.ascontiguousarray(w[::-1])
+    with torch.no_grad():
+        layer.weight.copy_(torch.from_numpy(w2))
+    assert torch.equal(layer(xt[:2]), y2)
+    layer.weights_changed()
+    y3 = layer(xt[:2])
+    assert np.array_equal(y3.cpu().numpy().view(np.uint32),
+                          oracle.forward(oracle_shape(oracle, d2), x[:2], w2)["dst"].view(np.uint32))
+    bw = layer.binarized_weights().cpu().numpy()
+    assert np.array_equal(np.signbit(bw), np.signbit(
+        oracle.binarize_weights_float(oracle_shape(oracle, d2), w2)))
+    # a stream other than the default one
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        y4 = layer(xt[:2])
+    side.synchronize()
+    assert torch.equal(y4, y3)
+
+
 def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
     """With the matrix-core kernel, calculate_k leaves the box filter to the convolution.
     The K plane must still be what calculate_k saw: (1) read back before any forward, (2)

@@ -186,3 +186,37 @@ def test_golden_workloads(oracle, golden, name):
     out = oracle.forward(oracle_shape(oracle, d), x, w)
     for key, want in g["sha256"].items():
         assert sha256(out[key]) == want, key
+
+
+def test_binarize_weights_float_closed_forms(oracle):
+    """sign(w) * mean(w) (reference src/binarize_weights_float.cpp:3-25): the mean is of the
+    weights themselves, not of their magnitudes; -0.0 counts as >= 0; the sum runs in index
+    order in float."""
+    s = oracle.shape(1, 4, 3, 5, 5, 3, 3, 1, 1, 1, 1)
+    n = 4 * 3 * 3 * 3
+    ones = np.ones(n, np.float32)
+    assert np.array_equal(oracle.binarize_weights_float(s, ones), ones)
+    # alternating +-c sums to exactly zero (n is even): the outputs are zeros whose sign is
+    # that of the weight
+    alt = np.where(np.arange(n) % 2 == 0, np.float32(0.75), np.float32(-0.75))
+    out = oracle.binarize_weights_float(s, alt)
+    assert np.all(out == 0) and np.array_equal(np.signbit(out), alt < 0)
+    # a negative zero is "not negative"
+    w = np.full(n, 2.0, np.float32)
+    w[5] = -0.0
+    w[6] = -1.0
+    out = oracle.binarize_weights_float(s, w)
+    mean = np.float32(np.float32((n - 2) * 2.0 - 1.0) * np.float32(1.0 / n))
+    want = np.full(n, mean, np.float32)
+    want[6] = -mean
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    # sequential float sum, then one multiply by 1.f/n: restated with numpy scalars
+    w = synth.normal(5, n, 0.05)
+    acc = np.float32(0)
+    for v in w:
+        acc = np.float32(acc + v)
+    mean = np.float32(acc * np.float32(1.0 / n))
+    want = np.where(w >= 0, mean, -mean).astype(np.float32)
+    assert np.array_equal(oracle.binarize_weights_float(s, w).view(np.uint32),
+                          want.view(np.uint32))
+    assert abs(float(mean) - float(np.mean(w.astype(np.float64)))) < 1e-7

@@ -56,3 +56,18 @@ def test_negative_zero_differs_between_upstream_algorithms(oracle, reflib):
     assert same_bytes(mine["dst"], ref["dst"])
     alg = reflib.forward(d, x, w, algorithm=capi.ALGORITHM_REFERENCE)
     assert not np.allclose(mine["dst"], alg["dst"], atol=1e-3, rtol=0)
+
+
+@pytest.mark.parametrize("name,mb", [("alexnet_conv4_mb256", 1), ("alexnet_conv2_mb128", 1),
+                                     ("vgg_512_mb32", 1)])
+def test_binarize_weights_float_on_one_thread(oracle, reflib, name, mb):
+    """The float sign(w)*mean(w) helper, bit for bit, with the reference held to one OpenMP
+    thread: its sum is a shared variable updated from a parallel loop without a reduction
+    (reference src/binarize_weights_float.cpp:17-19), so only that run is defined."""
+    d, _, w = synth.make_workload(name, mb)
+    want = reflib.binarize_weights_float(d, w, threads=1)
+    got = oracle.binarize_weights_float(oracle_shape(oracle, d), w)
+    assert same_bytes(got, want)
+    # one value m where w >= 0 and -m elsewhere
+    m = want[w >= 0][0]
+    assert np.all(want[w >= 0] == m) and np.all(want[w < 0] == -m)
