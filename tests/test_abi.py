@@ -149,6 +149,19 @@ def test_reference_algorithm_has_no_gpu_path():
     lib.xnor_nn_destroy_convolution(C.byref(c))
 
 
+def test_word_size_of_the_exported_layout():
+    """The export helpers hand out the reference's CPU layout, whose packed words are 16 bits
+    wide while IC*KH*KW < 32767 and 32 bits wide from there on (reference
+    src/implementation.cpp:17-22, src/convolution_traits.hpp:29-56)."""
+    lib = capi.load()
+    for ic, want in ((384, 2), (3640, 2), (3641, 4), (4000, 4)):
+        c = capi.ConvolutionDesc()
+        lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, 0, 2, 0,
+                                     1, 16, ic, 5, 5, 3, 3, 1, 1, 1, 1)
+        assert lib.xnor_nn_hip_canonical_bici(C.byref(c)) == want, ic
+        lib.xnor_nn_destroy_convolution(C.byref(c))
+
+
 def test_package_does_not_touch_the_oracle():
     """The oracle is test infrastructure: nothing under xnor_nn_amd/ may name it."""
     pkg = os.path.join(ROOT, "xnor_nn_amd")

@@ -499,6 +499,15 @@ def test_upstream_performance_programs_run_unchanged(gpu, exe):
     assert out.stdout.strip().endswith("success"), out.stdout[-500:]
 
 
+def test_device_info(gpu):
+    """xnor_nn_hip_device_info: compute units and clock of the current device, what the
+    benchmark prices the XNOR/popcount kernel's ceiling with."""
+    import ctypes as C
+    cus, khz = C.c_int(0), C.c_int(0)
+    assert capi.load().xnor_nn_hip_device_info(C.byref(cus), C.byref(khz)) == 0
+    assert cus.value == 256 and 1_000_000 <= khz.value <= 3_000_000, (cus.value, khz.value)
+
+
 def test_binarize_weights_float(oracle, gpu):
     """xnor_nn_binarize_weights_float on host and on device buffers: the signs follow
     w >= 0 exactly (a negative zero counts as positive), every magnitude is the same float,
