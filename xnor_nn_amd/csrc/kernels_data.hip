@@ -138,7 +138,7 @@ void binarize_tile(const float *__restrict__ x, uint32_t *__restrict__ bits,
         }
     };
 
-    // everything after the loads of round 0; t holds them on entry
+    // everything after the loads of the first pass over the slices (r = 0); t holds them
     auto process = [&](float (&t)[32], uint32_t tile) {
         const uint32_t p = tile * TILE + lane;
         if (wave == 0) chain[lane] = 0.f;
