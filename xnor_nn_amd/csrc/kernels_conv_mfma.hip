@@ -264,7 +264,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             if (first < 0) first = 0;
             if (last > 31) last = 31;
             if (last < first) return 0u;
-            return (uint32_t)(((1ull << (last + 1)) - 1) & ~((1ull << first) - 1));
+            return (0xFFFFFFFFu >> (31 - last)) & (0xFFFFFFFFu << first);
         };
         rowmask[ps] = live[ps] ? run_of_bits(-ih0, g.ih - 1 - ih0) : 0u;
         colmask[ps] = run_of_bits(-iw0, g.iw - 1 - iw0);
@@ -290,10 +290,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     if (fuse_k && tid < nrows) a_early = a_plane[lo + tid];
     table[tid] = fp4_of_byte(tid);
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
-    {
-        const int oc = chunk * NT + tid;
-        alpha_lds[tid] = oc < g.oc ? alpha[oc] : 0.f;
-    }
+    // asked for now, put into LDS after the expansion: nothing needs it before the epilogue,
+    // and the first barrier does not have to wait for it
+    const float alpha_early = chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
     if (fuse_k) { // mean|x| of the staged input pixels, plus one slot that holds zero
         if (tid < nrows) a_lds[tid] = a_early;
         if (tid == 0) a_lds[max_rows] = 0.f;
@@ -361,6 +360,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
             if (i < nitems) expand(i, w[u]);
         }
     }
+
+    alpha_lds[tid] = alpha_early;
 
     // ---- this wave: 64 filters x 32*PS pixels --------------------------------------------------
     const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
