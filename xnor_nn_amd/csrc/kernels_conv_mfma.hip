@@ -852,13 +852,21 @@ size_t lds_bytes(const Geometry &g, int ps) {
     return bytes;
 }
 
-// 32-pixel blocks per tile.  Cost of a choice = (waves the busiest SIMD runs one after the
-// other) x (work per wave, plus half a block for the staging and epilogue every tile pays).
-// With few waves per SIMD the busiest one sets the pace, so the count is rounded up; with
-// many, the hardware's dynamic scheduling evens the load out.  Ties go to the larger tile,
-// which streams fewer weight bytes.  (Measured on MI355X, PS 1/2/3/4: conv4 MB 256 = 34.7 /
-// 27.0 / 26.6 / 27.5 us, ResNet 3x3 MB 64 = 113 / 97.0 / 96.6 / 96.9, VGG 512 MB 32 = 49.2 /
-// 37.6 / 39.6 / 35.2, conv2 shape MB 128 = 58.2 / 46.3 / 45.5 / 44.3.)
+// 32-pixel blocks per tile, by a model of the kernel's time in core cycles that was fitted to
+// measurements on MI355X (conv4 from MB 4 to MB 1024, ResNet 3x3 56x56 MB 1 to 64, VGG 512 MB
+// 1 to 32, the conv2 shape, 64- and 128-channel layers; PS 1/2/3/4 at conv4 MB 256 = 34.7 /
+// 27.0 / 26.6 / 27.5 us, at MB 32 = 8.2 / 9.4 / 11.7 / 13.8 us).
+//   one wave:   staging (set-up, plus 264 cycles per 256 packed words to expand)
+//               + PS x (epilogue 1700 + 64 per step of the main loop)
+//               -- with one pixel block and more than one wave per SIMD a step costs as much
+//               as with two: the weight stream (2 KB per wave and step whatever the tile)
+//               sets its pace, not the matrix instructions;
+//   the kernel: one wave's time for the first wave of the busiest SIMD, 0.35 of it more for
+//               the second (the phases of two resident waves overlap), 0.75 for every further
+//               one; with few waves per SIMD the busiest one counts (rounded up), with many
+//               the hardware's dynamic scheduling evens the load out;
+//   a tile that needs more than half the LDS runs alone on its CU: 15 % more.
+// Ties go to the larger tile, which streams fewer weight bytes.
 // Four pixel blocks do not fit the register file with 16 steps per tap or with tap pairing
 // over five words (those variants spill), and are not instantiated for channel parts.
 bool tile_fits_registers(const Geometry &g, int ps) {
@@ -876,6 +884,8 @@ int pick_ps(const Geometry &g) {
     const int chunks = (g.oc + NT - 1) / NT;
     const int waves_per_block = g.oc >= NT ? 4 : (g.oc + 63) / 64;
     const double simds = (double)g.cus * 4;
+    const int units = pair_taps(g) ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw * channel_parts(g);
+    const double steps_total = (double)units * steps_per_tap(g);
     int best = 0;
     double best_cost = 0;
     for (int ps = 4; ps >= 1; ps--) {
@@ -883,14 +893,15 @@ int pick_ps(const Geometry &g) {
         if (!tile_fits_registers(g, ps)) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
         const double per_simd = tiles * chunks * waves_per_block / simds;
-        const double busiest = per_simd <= 4 ? (double)(long)(per_simd + 0.999999)
-                                             : per_simd + 0.5;
-        // a tile that needs more than half the LDS runs alone on its CU: nothing covers its
-        // staging and its epilogue
+        const double busiest = per_simd <= 1 ? 1.0
+            : per_simd <= 4 ? (double)(long)(per_simd + 0.999999) : per_simd + 0.5;
+        const double words = (double)max_tile_rows(g, 32 * ps) * g.xw;
+        const double stream_bound = ps < 2 && per_simd > 1 ? 2.0 : (double)ps;
+        const double wave = 3700.0 + 264.0 * words / 256.0 + 1700.0 * ps
+            + 64.0 * steps_total * stream_bound;
+        const double waves = busiest < 2 ? 1.0 : 1.35 + 0.75 * (busiest - 2.0);
         const double alone = lds_bytes(g, ps) > (size_t)LDS_TWO_PER_CU ? 1.15 : 1.0;
-        // below two blocks the weight stream (2 KB per wave and step whatever the tile) sets
-        // the pace of a step, not the matrix instructions
-        const double cost = (busiest < 1 ? 1 : busiest) * ((ps < 2 ? 2 : ps) + 0.5) * alone;
+        const double cost = wave * waves * alone;
         if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
     }
     return best;
