@@ -71,7 +71,10 @@ constexpr int ALPHA_CHUNK = 512;
 __global__ __launch_bounds__(64)
 void alpha_oihw_kernel(const float *__restrict__ w, float *__restrict__ alpha, const int oc_n,
         const int n, const float chw) {
-    __shared__ float tile[ALPHA_F][ALPHA_CHUNK + 1];
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    // rows of ALPHA_CHUNK + 4 floats: 16-byte aligned, and the eight summing lanes start four
+    // banks apart, so their 16-byte reads do not collide
+    __shared__ __attribute__((aligned(16))) float tile[ALPHA_F][ALPHA_CHUNK + 4];
     constexpr int PER_LANE = ALPHA_CHUNK / 64;
     const int lane = threadIdx.x;
     const int f0 = blockIdx.x * ALPHA_F;
@@ -98,13 +101,27 @@ void alpha_oihw_kernel(const float *__restrict__ w, float *__restrict__ alpha, c
         __syncthreads();
         // Elements past the end of the row were stored as +0, and s + 0 == s for these
         // non-negative sums, so whole batches can be read before they are added in order.
+        // Two register sets of 16 values: one is read from LDS while the other is added.
         if (lane < ALPHA_F) {
-            for (int j = 0; j < ALPHA_CHUNK; j += 16) {
-                float v[16];
+            const v4f *row = reinterpret_cast<const v4f *>(tile[lane]);
+            v4f a[4], b[4];
 #pragma unroll
-                for (int u = 0; u < 16; u++) v[u] = tile[lane][j + u];
+            for (int u = 0; u < 4; u++) a[u] = row[u];
+            for (int j = 0; j < ALPHA_CHUNK / 16; j += 2) {
 #pragma unroll
-                for (int u = 0; u < 16; u++) acc = __fadd_rn(acc, v[u]);
+                for (int u = 0; u < 4; u++) b[u] = row[4 * (j + 1) + u];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc = __fadd_rn(acc, a[u][e]);
+                if (j + 2 < ALPHA_CHUNK / 16) {
+#pragma unroll
+                    for (int u = 0; u < 4; u++) a[u] = row[4 * (j + 2) + u];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc = __fadd_rn(acc, b[u][e]);
             }
         }
         __syncthreads();
