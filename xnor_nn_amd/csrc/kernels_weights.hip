@@ -43,22 +43,9 @@ void pack_weights_kernel(const float *__restrict__ w, uint32_t *__restrict__ bit
 }
 
 // alpha[oc] = sum over (ic, kh, kw), nested in that order, of fl(|w| * chw)
-// (reference src/bcast_binarize_weights.cpp:95-115).  One thread per filter, any layout.
-__global__ __launch_bounds__(64)
-void alpha_kernel(const float *__restrict__ w, float *__restrict__ alpha,
-        const Geometry g, const float chw) {
-    const int oc = blockIdx.x * blockDim.x + threadIdx.x;
-    if (oc >= g.oc) return;
-    float acc = 0.f;
-    for (int ic = 0; ic < g.ic; ic++)
-        for (int kh = 0; kh < g.kh; kh++)
-            for (int kw = 0; kw < g.kw; kw++)
-                acc = __fadd_rn(acc,
-                        __fmul_rn(__builtin_fabsf(w[w_index(g, oc, ic, kh, kw)]), chw));
-    alpha[oc] = acc;
-}
-
-// The same sum for OIHW weights, where a filter is one contiguous row of n = IC*KH*KW floats
+// (reference src/bcast_binarize_weights.cpp:95-115): two kernels, one per weight layout.
+//
+// OIHW weights: a filter is one contiguous row of n = IC*KH*KW floats
 // already in summation order.  One wave per ALPHA_F filters.  The rows are read ALPHA_CHUNK
 // elements at a time with coalesced loads (all lanes read consecutive elements of one
 // filter), passed through LDS and summed in order by lane f for filter f; the loads of the
@@ -133,6 +120,63 @@ void alpha_oihw_kernel(const float *__restrict__ w, float *__restrict__ alpha, c
     if (lane < nf) alpha[f0 + lane] = acc;
 }
 
+// Weights in which the filters are the contiguous index (HWIO): element t of
+// the summation order (t = (ic*KH + kh)*KW + kw) of 64 consecutive filters is one coalesced
+// load, a lane is a filter.  With one wave per 64 filters and a load per addition the kernel
+// waited for memory 3456 times in a row (800 us for 256 x 3456 weights); here eight waves
+// fetch the next ALPHA_T elements into registers while wave 0 adds the current ones, in
+// order, out of LDS.
+constexpr int ALPHA_T = 256;
+
+__global__ __launch_bounds__(512)
+void alpha_strided_kernel(const float *__restrict__ w, float *__restrict__ alpha,
+        const Geometry g, const float chw, const FastDiv div_taps, const FastDiv div_kw) {
+    __shared__ float tile[ALPHA_T][64];
+    constexpr int PER_WAVE = ALPHA_T / 8;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int oc = blockIdx.x * 64 + lane;
+    const int ocl = oc < g.oc ? oc : g.oc - 1;
+    const int taps = g.kh * g.kw, n = g.ic * taps;
+    float next[PER_WAVE];
+    auto fetch = [&](int c) { // this wave's rows of chunk c: t = c*ALPHA_T + wave*PER_WAVE + u
+#pragma unroll
+        for (int u = 0; u < PER_WAVE; u++) {
+            const int t = c * ALPHA_T + wave * PER_WAVE + u; // wave-uniform
+            const int tc = t < n ? t : n - 1;
+            const int ic = (int)div_taps.div((uint32_t)tc), tap = tc - ic * taps;
+            const int kh = (int)div_kw.div((uint32_t)tap), kw = tap - kh * g.kw;
+            const float v = w[w_index(g, ocl, ic, kh, kw)];
+            next[u] = t < n ? __fmul_rn(__builtin_fabsf(v), chw) : 0.f; // +0 adds nothing
+        }
+    };
+    auto publish = [&]() {
+#pragma unroll
+        for (int u = 0; u < PER_WAVE; u++) tile[wave * PER_WAVE + u][lane] = next[u];
+    };
+    const int chunks = (n + ALPHA_T - 1) / ALPHA_T;
+    float acc = 0.f;
+    fetch(0);
+    publish();
+    __syncthreads();
+    for (int c = 0; c < chunks; c++) {
+        if (c + 1 < chunks) fetch(c + 1);
+        if (wave == 0) {
+            for (int r = 0; r < ALPHA_T; r += 16) {
+                float v[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) v[u] = tile[r + u][lane];
+#pragma unroll
+                for (int u = 0; u < 16; u++) acc = __fadd_rn(acc, v[u]);
+            }
+        }
+        __syncthreads(); // the chunk has been added: its rows may be overwritten
+        if (c + 1 < chunks) publish();
+        __syncthreads();
+    }
+    if (wave == 0 && oc < g.oc) alpha[oc] = acc;
+}
+
 // opc[oh][ow] = IC * number of in-bounds taps (reference
 // src/bcast_binarize_weights.cpp:126-142).
 __global__ __launch_bounds__(256)
@@ -191,7 +235,9 @@ hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *
                 s, w, alpha,
                 g.oc, g.ic * g.kh * g.kw, chw);
     else
-        hipLaunchKernelGGL(alpha_kernel, dim3((g.oc + 63) / 64), dim3(64), 0, s, w, alpha, g, chw);
+        hipLaunchKernelGGL(alpha_strided_kernel, dim3((g.oc + 63) / 64), dim3(512), 0, s, w,
+                alpha, g, chw, FastDiv::make((uint32_t)(g.kh * g.kw)),
+                FastDiv::make((uint32_t)g.kw));
     hipLaunchKernelGGL(op_count_kernel, dim3((g.ohw + 255) / 256), dim3(256), 0, s, opc, g);
     return hipGetLastError();
 }
