@@ -22,8 +22,28 @@ extern "C" {
 /* HIP stream (a hipStream_t passed as void*) on which the executors of this descriptor
  * launch; default: the null stream.  With device pointers in slots 0..2 the executors
  * only enqueue work and return; with host pointers they copy synchronously.
- * Stands in for the reference's implicit "runs on the calling thread + OpenMP team". */
+ * Stands in for the reference's implicit "runs on the calling thread + OpenMP team".
+ * Threads: as in the reference (src/bcast_convolution.hpp:77-93) the executors keep nothing
+ * between calls but the launch plan, so several host threads may run one descriptor, each
+ * with a resource table of its own; calls on one descriptor are serialised internally (they
+ * share its stream and, for host pointers, its staging buffers). */
 xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *stream);
+
+/* Stage fusion, on by default.  The reference's three per-forward stages each make a full
+ * pass of their own (reference src/bcast_binarize_data.cpp:43-73,
+ * src/bcast_calculate_k.cpp:42-85).  Here binarize_data also leaves mean|x| in res[a], and
+ * the calculate_k that follows it immediately on the same res[user_src] and res[a] does not
+ * read the input again; with the matrix-core convolution calculate_k also leaves its box
+ * filter to forward, which sums K on the fly and stores the K plane.  What is handed over is
+ * recorded against the device buffers of the resource table, so calls on other tables do
+ * not interfere; any other executor on the table, freeing the table or destroying the
+ * descriptor withdraws it.  A caller that changes the contents of user_src between
+ * binarize_data and calculate_k, or that reads res[k] as a raw device pointer between
+ * calculate_k and forward, switches fusion off (on = 0; the environment variable
+ * XNOR_NN_HIP_SEPARATE_K=1 does the same for every descriptor): every executor then
+ * completes its own stage as in the reference.  xnor_nn_hip_export_floats always returns
+ * the finished K plane. */
+xnor_nn_status_t xnor_nn_hip_set_stage_fusion(const xnor_nn_convolution_t *c, int on);
 
 /* Block until everything enqueued by this descriptor's executors has finished. */
 xnor_nn_status_t xnor_nn_hip_synchronize(const xnor_nn_convolution_t *c);
@@ -62,7 +82,9 @@ xnor_nn_status_t xnor_nn_hip_export_operations_count(const xnor_nn_convolution_t
 /* Run the convolution stage but store the raw integer accumulators
  * popc[mb][oc][oh][ow] (int32, host or device pointer) instead of the scaled floats:
  * the `d_arr` values of reference src/default/bcast_convolution_default.cpp:64-91.
- * Needs res[bin_src] and res[bin_weights]; same kernel as forward, other epilogue. */
+ * Needs res[bin_src] and res[bin_weights] only (the operation count that turns the
+ * matrix-core kernel's 2*popc - n back into popc is derived from the geometry inside the
+ * kernel); same kernel as forward, other epilogue. */
 xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
         xnor_nn_resources_t res, int32_t *popc);
 

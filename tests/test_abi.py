@@ -184,3 +184,38 @@ def test_upstream_examples_compile_and_link_unchanged(tmp_path, name, cc):
     subprocess.check_call([cc, "-I", INCLUDE, os.path.join("/root/reference/example", name),
                            "-L", libdir, "-lxnor_nn", "-Wl,-rpath," + libdir,
                            "-Wl,-rpath-link,/opt/rocm/lib", "-o", str(exe)])
+
+
+def test_forward_popcount_needs_only_the_two_packed_tensors():
+    """xnor_nn_hip_forward_popcount checks exactly the slots its header names: bin_src,
+    bin_weights and the output pointer (host-only: the checks come before device work)."""
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, capi.FMT_NCHW,
+                                 capi.FMT_OIHW, capi.FMT_NCHW, 1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1)
+    res = capi.Resources()
+    out = (C.c_int32 * (16 * 25))()
+    assert lib.xnor_nn_hip_forward_popcount(C.byref(c), res, out) == capi.ERROR_INVALID_INPUT
+    dummy = (C.c_float * 4)()
+    res[capi.RES_BIN_SRC] = C.addressof(dummy)
+    assert lib.xnor_nn_hip_forward_popcount(C.byref(c), res, out) == capi.ERROR_INVALID_INPUT
+    res[capi.RES_BIN_WEIGHTS] = C.addressof(dummy)
+    assert lib.xnor_nn_hip_forward_popcount(C.byref(c), res, None) == capi.ERROR_INVALID_INPUT
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+    # a descriptor without the bcast state has no popcount path
+    assert lib.xnor_nn_hip_forward_popcount(C.byref(c), res, out) == capi.ERROR_INVALID_INPUT
+    assert lib.xnor_nn_hip_set_stage_fusion(C.byref(c), 0) == capi.ERROR_INVALID_INPUT
+
+
+def test_stage_fusion_switch_and_table_bookkeeping_without_a_gpu():
+    """The switch is per descriptor; freeing a zeroed or hand-filled table and destroying a
+    descriptor that never ran are safe (the hand-over bookkeeping is keyed on buffers)."""
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, capi.FMT_NCHW,
+                                 capi.FMT_OIHW, capi.FMT_NCHW, 1, 16, 8, 5, 5, 3, 3, 1, 1, 1, 1)
+    assert lib.xnor_nn_hip_set_stage_fusion(C.byref(c), 0) == capi.SUCCESS
+    assert lib.xnor_nn_hip_set_stage_fusion(C.byref(c), 1) == capi.SUCCESS
+    res = capi.Resources()
+    lib.xnor_nn_free_resources(res)
+    lib.xnor_nn_destroy_convolution(C.byref(c))

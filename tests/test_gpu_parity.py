@@ -573,6 +573,21 @@ def test_pytorch_layer(oracle, gpu):
         y4 = layer(xt[:2])
     side.synchronize()
     assert torch.equal(y4, y3)
+    # first call and a weight change both inside a side stream: the weight stage has to run on
+    # that stream too, behind the copy into `weight` and ahead of the forward pass
+    layer2 = XnorConv2d(d["ic"], d["oc"], (d["kh"], d["kw"]), stride=(d["sh"], d["sw"]),
+                        padding=(d["ph"], d["pw"]), weight=torch.from_numpy(w)).to(gpu)
+    w2t = torch.from_numpy(w2).to(gpu)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        ya = layer2(xt[:2])
+        layer2.weight.data.copy_(w2t, non_blocking=True)
+        layer2.weights_changed()
+        yb = layer2(xt[:2])
+        bw2 = layer2.binarized_weights()
+    side.synchronize()
+    assert torch.equal(ya, y2) and torch.equal(yb, y3)
+    assert np.array_equal(bw2.cpu().numpy(), bw)
 
 
 def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
@@ -637,3 +652,55 @@ def test_linearity_of_scaling_at_full_size(gpu):
     assert np.array_equal(conv.export_bin_src(), b1)
     assert torch.equal(y2, y1 * 2)
     conv.close()
+
+
+def test_random_problems_until_the_time_is_up(oracle):
+    """Fifteen seconds of seeded random problems larger than the ones above (channel counts
+    around the 32/64/1024 boundaries up to 2048, kernels 1..9, strides 1..4, paddings 0..4,
+    images up to 43 x 43, every layout combination, inputs with exact zeros of both signs):
+    dst and the raw popcounts against the oracle, bit for bit, stopping at the first
+    mismatch."""
+    import time
+    rng = np.random.default_rng(20251)
+    t_end = time.time() + 15.0
+    n = 0
+    while time.time() < t_end:
+        kh, kw = int(rng.integers(1, 10)), int(rng.integers(1, 10))
+        ph, pw = int(rng.integers(0, 5)), int(rng.integers(0, 5))
+        sh, sw = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        ih = int(rng.integers(max(1, kh - 2 * pw), 44))
+        iw = int(rng.integers(max(1, kw - 2 * pw), 44))
+        ic = int(rng.choice([1, 3, 4, 31, 32, 33, 64, 65, 96, 100, 128, 160, 200, 256, 257, 320,
+                             384, 448, 512, 513, 640, 700, 1000, 1024, 1028, 1500, 2048]))
+        oc = int(rng.choice([1, 7, 16, 31, 32, 33, 64, 65, 100, 128, 130, 256, 260, 384, 512,
+                             600]))
+        mb = int(rng.integers(1, 7))
+        oh, ow = (ih + 2 * pw - kh) // sh + 1, (iw + 2 * pw - kw) // sw + 1
+        if oh < 1 or ow < 1 or ih + 2 * ph < kh:
+            continue
+        if max(mb * ic * ih * iw, mb * oc * oh * ow, oc * ic * kh * kw) > 6e6:
+            continue
+        if mb * oc * oh * ow * ic * kh * kw > 4e10:
+            continue
+        fmts = (int(rng.choice([capi.FMT_NCHW, capi.FMT_NHWC])),
+                int(rng.choice([capi.FMT_OIHW, capi.FMT_HWIO])),
+                int(rng.choice([capi.FMT_NCHW, capi.FMT_NHWC])))
+        d = dict(mb=mb, ic=ic, oc=oc, ih=ih, iw=iw, kh=kh, kw=kw, sh=sh, sw=sw, ph=ph, pw=pw)
+        x = synth.normal(1000 + n, mb * ic * ih * iw).reshape(mb, ic, ih, iw)
+        x.ravel()[::7] = 0.0
+        x.ravel()[3::11] = -0.0
+        w = synth.normal(5000 + n, oc * ic * kh * kw, 0.05).reshape(oc, ic, kh, kw)
+        xs = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if fmts[0] == capi.FMT_NHWC else x
+        ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
+        want = oracle.forward(oracle_shape(oracle, d, fmts), xs, ws)
+        print("case", n, d, fmts, flush=True)
+        conv = make(d, ws, fmts)
+        dst = np.empty(want["dst"].shape, np.float32)
+        conv.forward(xs, dst)
+        ok = np.array_equal(dst.view(np.uint32), want["dst"].view(np.uint32)) \
+            and np.array_equal(conv.forward_popcount(), want["popc"])
+        name = conv.kernel_name(0)
+        conv.close()
+        assert ok, "case %d %s formats %s (%s)" % (n, d, fmts, name)
+        n += 1
+    assert n >= 5

@@ -1,12 +1,20 @@
-"""Static check of the matrix-core convolution's machine code (no GPU needed).
+"""Static check of hand-scheduled machine code (no GPU needed).
 
-The kernel starts its vector memory loads by hand and waits for them later with s_waitcnt
-vmcnt(N).  Between the load and the wait that covers it, the destination registers hold stale
-data and the hardware will still write them: any other instruction that reads or writes such a
-register in that window is a bug the compiler cannot see (it takes the inline-asm load for an
-ordinary definition), and the symptom is a wrong result or a wild address on the GPU.  The test
-compiles the kernel file to ISA and walks every path of every kernel's control flow graph with
-the queue of loads in flight."""
+The matrix-core convolution starts its vector memory loads and its LDS reads by hand and waits
+for them later with s_waitcnt vmcnt(N) / lgkmcnt(N).  Between a load and the wait that covers
+it, the destination registers hold stale data and the hardware will still write them: any
+other instruction that reads or writes such a register in that window is a bug the compiler
+cannot see (it takes the inline-asm load for an ordinary definition), and the symptom is a
+wrong result or a wild address on the GPU.  The test compiles the kernel files to ISA and
+walks every path of every kernel's control flow graph with the queues of loads in flight:
+vector memory (loads and stores, which return in order and share vmcnt) and LDS (reads and
+writes; LDS operations complete in order among themselves, so after lgkmcnt(N) all but the
+newest N of them are done whatever scalar memory loads share the counter).
+
+Only the matrix-core kernel is walked.  The streaming kernels of stages 1 and 2 issue their
+buffer loads through compiler builtins, so the compiler's own wait insertion covers them; a
+walk that knows nothing about branch conditions reports paths there that cannot be taken
+(a wave that skips its turn in the ordered hand-over of the running sum)."""
 import os
 import re
 import subprocess
@@ -16,12 +24,8 @@ import pytest
 from xnor_nn_amd import build
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SOURCE = os.path.join(ROOT, "xnor_nn_amd", "csrc", "kernels_conv_mfma.hip")
-
-# Variants the host never launches because they do not fit the register file (pick_ps in the
-# kernel file): 4 pixel blocks with 16 steps per tap, or with tap pairing over 5 words.  Their
-# spill code moves registers around while loads are in flight.
-NEVER_LAUNCHED = re.compile(r"conv_mfma_fp4_kernelILi(16ELi4ELb[01]ELb0|5ELi4ELb[01]ELb1)E")
+CSRC = os.path.join(ROOT, "xnor_nn_amd", "csrc")
+VM_MAX, LGKM_MAX = 64, 16
 
 
 def vgprs(token):
@@ -34,96 +38,154 @@ def vgprs(token):
 
 
 def parse(body):
-    """One tuple per line: (kind, registers touched, load destination, vmcnt, branch target)."""
+    """One tuple per line: (kind, registers touched, vector-memory destination, LDS
+    destination, (vmcnt, lgkmcnt), branch target); a destination of frozenset() is an
+    operation that counts without writing a register (a store, an LDS write)."""
     label_at = {l[:-1]: i for i, l in enumerate(body) if l.startswith(".LBB")}
     out = []
     for line in body:
         if line.startswith(".LBB"):
-            out.append(("label", None, None, None, None))
+            out.append(("label", None, None, None, None, None))
             continue
         op = line.split()[0]
         ops = [o for o in re.split(r"[ ,]+", line)[1:] if o]
         if op == "s_endpgm":
-            out.append(("end", None, None, None, None))
+            out.append(("end", None, None, None, None, None))
         elif op == "s_waitcnt":
-            m = re.search(r"vmcnt\((\d+)\)", line)
-            out.append(("wait", None, None, int(m.group(1)) if m else None, None))
+            vm = re.search(r"vmcnt\((\d+)\)", line)
+            lg = re.search(r"lgkmcnt\((\d+)\)", line)
+            out.append(("wait", None, None, None,
+                        (int(vm.group(1)) if vm else None, int(lg.group(1)) if lg else None),
+                        None))
         elif op.startswith("s_cbranch") or op == "s_branch":
-            out.append(("jump" if op == "s_branch" else "branch", None, None, None,
+            out.append(("jump" if op == "s_branch" else "branch", None, None, None, None,
                         label_at.get(ops[-1])))
         elif op.startswith("s_"):
-            out.append(("scalar", None, None, None, None))
+            out.append(("scalar", None, None, None, None, None))
         else:
             touched = frozenset().union(*[vgprs(o) for o in ops]) if ops else frozenset()
-            dst = None
-            if re.match(r"(buffer|global|scratch)_load", op):
-                dst = vgprs(ops[0])
-            elif re.match(r"(buffer|global|scratch)_store", op):
-                dst = frozenset()  # stores count in vmcnt as well
-            out.append(("vector", touched, dst, None, None))
+            vdst = ldst = None
+            if re.match(r"(buffer|global|scratch|flat)_load", op):
+                vdst = vgprs(ops[0])
+                if op.startswith("flat"):
+                    ldst = vdst  # a flat load counts in both
+            elif re.match(r"(buffer|global|scratch|flat)_(store|atomic)", op):
+                vdst = frozenset()  # stores count in vmcnt as well
+            elif op.startswith("ds_"):
+                ldst = frozenset() if re.match(r"ds_(write|add|sub|min|max|and|or|xor)", op) \
+                    and "_rtn" not in op else vgprs(ops[0])
+            out.append(("vector", touched, vdst, ldst, None, None))
     return out
 
 
-def hazards_of(body):
-    """body: instructions and .LBB labels of one kernel, in layout order."""
-    first = next((i for i, l in enumerate(body) if l.startswith("buffer_load_dwordx4")), None)
-    if first is None:
-        return None
+def hazards_of(body, first=0):
+    """body: instructions and .LBB labels of one kernel, in layout order; the walk starts at
+    instruction `first` with nothing in flight.
+
+    State: for every register with a load on the way, how many operations of the same queue
+    have been issued since (its age).  s_waitcnt with count N completes everything of age >= N;
+    the counters have 6 and 4 bits, so the hardware itself holds an instruction back until
+    fewer than 64 vector memory / 16 LDS operations are in flight, and whatever is older has
+    completed.  Where paths meet (labels), a register keeps the smaller of its ages: the walk
+    is a fixed-point iteration over the control flow graph, conservative where paths differ."""
     code = parse(body)
-    seen, work, bad = set(), [(first, ())], set()
+    at_label, work, bad = {}, [(first, {}, {})], set()
+
+    def issue(ages, dst, limit):
+        ages = {r: a + 1 for r, a in ages.items() if a + 1 < limit}
+        for r in dst:
+            ages[r] = 0
+        return ages
+
+    def join(old, new):
+        out = dict(old)
+        for r, a in new.items():
+            out[r] = min(a, out.get(r, a))
+        return out
+
     while work:
-        pc, queue = work.pop()  # queue: destination registers of the loads in flight, oldest first
-        in_flight = frozenset().union(*queue) if queue else frozenset()
+        pc, vm_age, lds_age = work.pop()
         while pc < len(code):
-            kind, touched, dst, vm, target = code[pc]
+            kind, touched, vdst, ldst, counts, target = code[pc]
             if kind == "label":
-                if (pc, queue) in seen:
-                    break
-                seen.add((pc, queue))
+                if pc in at_label:
+                    merged = (join(at_label[pc][0], vm_age), join(at_label[pc][1], lds_age))
+                    if merged == at_label[pc]:
+                        break
+                    at_label[pc] = merged
+                    vm_age, lds_age = merged
+                else:
+                    at_label[pc] = (dict(vm_age), dict(lds_age))
             elif kind == "end":
                 break
             elif kind == "wait":
-                if vm is not None and len(queue) > vm:
-                    queue = queue[len(queue) - vm:] if vm else ()
-                    in_flight = frozenset().union(*queue) if queue else frozenset()
+                vm, lg = counts
+                if vm is not None:
+                    vm_age = {r: a for r, a in vm_age.items() if a < vm}
+                if lg is not None:
+                    lds_age = {r: a for r, a in lds_age.items() if a < lg}
             elif kind in ("branch", "jump"):
                 if target is not None:
-                    work.append((target, queue))
+                    work.append((target, dict(vm_age), dict(lds_age)))
                 if kind == "jump":
                     break
             elif kind == "vector":
-                if touched & in_flight:
+                if any(r in vm_age or r in lds_age for r in touched):
                     bad.add((pc, body[pc]))
-                if dst is not None:
-                    queue = queue + (dst,)
-                    in_flight = in_flight | dst
+                if vdst is not None:
+                    vm_age = issue(vm_age, vdst, VM_MAX)
+                if ldst is not None:
+                    lds_age = issue(lds_age, ldst, LGKM_MAX)
             pc += 1
     return sorted(bad)
 
 
-@pytest.fixture(scope="module")
-def isa(tmp_path_factory):
-    out = tmp_path_factory.mktemp("isa") / "kernels_conv_mfma.s"
+def compile_to_isa(tmp, name):
+    out = tmp / (name + ".s")
+    source = os.path.join(CSRC, name + ".hip")
     cmd = [build.hipcc()] + [f for f in build.FLAGS if f not in ("-shared", "-fPIC")] + [
-        "-S", "--cuda-device-only", "-I" + os.path.join(ROOT, "include"),
-        "-I" + os.path.dirname(SOURCE), SOURCE, "-o", str(out)]
+        "-S", "--cuda-device-only", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, source,
+        "-o", str(out)]
     subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
     return out.read_text().split("\n")
 
 
-def test_no_register_is_touched_while_its_load_is_in_flight(isa):
-    starts = [i for i, l in enumerate(isa) if re.match(r"^_ZN\S*conv_mfma_fp4_kernel\S*:", l)]
-    assert len(starts) >= 90
-    checked = 0
-    for st in starts:
-        if NEVER_LAUNCHED.search(isa[st]):
-            continue
+def kernels_of(isa, pattern):
+    """(mangled name, instructions and labels) of every kernel whose symbol matches."""
+    for st in [i for i, l in enumerate(isa) if re.match(pattern, l)]:
         end = next(i for i in range(st, len(isa)) if ".end_amdhsa_kernel" in isa[i])
         body = [l.strip().split(";")[0].rstrip() for l in isa[st:end]]
-        body = [l for l in body if l and (not l.startswith(".") or l.startswith(".LBB"))]
-        bad = hazards_of(body)
-        assert bad is not None, "no fragment loads found in " + isa[st]
+        yield isa[st], [l for l in body if l and (not l.startswith(".") or l.startswith(".LBB"))]
+
+
+def test_no_register_is_touched_while_its_load_is_in_flight(tmp_path):
+    """Every variant of the matrix-core kernel that the library holds (all of them can be
+    launched), from its first hand-issued fragment load to the end."""
+    isa = compile_to_isa(tmp_path, "kernels_conv_mfma")
+    checked = 0
+    for name, body in kernels_of(isa, r"^_ZN\S*conv_mfma_fp4_kernel\S*:"):
+        first = next((i for i, l in enumerate(body) if l.startswith("buffer_load_dwordx4")),
+                     None)
+        assert first is not None, "no fragment loads found in " + name
+        bad = hazards_of(body, first)
         assert not bad, "%s: %d instructions touch a register whose load is in flight, " \
-            "first: %s" % (isa[st][:90], len(bad), bad[0][1])
+            "first: %s" % (name[:90], len(bad), bad[0][1])
         checked += 1
-    assert checked >= 80
+    assert checked >= 90
+
+
+def test_the_walker_sees_a_planted_hazard():
+    """The checker itself: a register read one instruction before the wait that covers its
+    load, for a vector memory load and for an LDS read, and the same code with the wait in
+    place."""
+    ok = ["buffer_load_dwordx4 v[4:7], v1, s[0:3], 0 offen", "ds_read_b128 v[8:11], v2",
+          "s_waitcnt vmcnt(0) lgkmcnt(0)", "v_add_u32_e32 v3, v4, v8", "s_endpgm"]
+    assert hazards_of(ok) == []
+    early_vm = [ok[0], ok[1], "s_waitcnt lgkmcnt(0)", ok[3], ok[4]]
+    assert [b[1] for b in hazards_of(early_vm)] == [ok[3]]
+    early_lds = [ok[0], ok[1], "s_waitcnt vmcnt(0)", ok[3], ok[4]]
+    assert [b[1] for b in hazards_of(early_lds)] == [ok[3]]
+    # in-order return: with one operation allowed in flight the older of two is done
+    two = ["ds_read_b128 v[4:7], v2", "ds_read_b128 v[8:11], v2 offset:16",
+           "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v0, v4", "v_mov_b32_e32 v1, v8", "s_endpgm"]
+    assert [b[1] for b in hazards_of(two)] == ["v_mov_b32_e32 v1, v8"]

@@ -71,3 +71,38 @@ def test_binarize_weights_float_on_one_thread(oracle, reflib, name, mb):
     # one value m where w >= 0 and -m elsewhere
     m = want[w >= 0][0]
     assert np.all(want[w >= 0] == m) and np.all(want[w < 0] == -m)
+
+
+LAYOUTS = [(s, w, o) for s in (capi.FMT_NCHW, capi.FMT_NHWC)
+           for w in (capi.FMT_OIHW, capi.FMT_HWIO) for o in (capi.FMT_NCHW, capi.FMT_NHWC)]
+
+
+@pytest.mark.parametrize("fmts", LAYOUTS, ids=lambda f: "%d%d%d" % f)
+@pytest.mark.parametrize("t", [
+    (2, 32, 16, 6, 5, 3, 3, 1, 1, 1, 1),       # one full word, filters = one block
+    (3, 40, 32, 9, 11, 3, 3, 1, 1, 1, 1),      # ragged channel tail
+    (2, 96, 48, 13, 13, 5, 5, 1, 1, 2, 2),     # conv2-like: three words, 5 x 5
+    (1, 70, 64, 7, 5, 3, 3, 2, 2, 1, 1),       # stride 2, odd byte count (pad byte)
+], ids=shapes.shape_id)
+def test_every_layout_combination(oracle, reflib, t, fmts):
+    """NHWC input, HWIO weights and NHWC output in all eight combinations (reference
+    src/bcast_binarize_data.cpp:56-57, src/bcast_calculate_k.cpp:59-60,
+    src/bcast_binarize_weights.cpp:71-72, src/default/bcast_convolution_default.cpp:97-99):
+    the oracle's layout branches against the compiled reference, all seven tensors."""
+    d = shapes.as_dims(t)
+    x = synth.normal(131, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::6] = 0.0
+    x.ravel()[1::8] = -0.0
+    w = synth.normal(132, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    if fmts[0] == capi.FMT_NHWC:
+        x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    if fmts[1] == capi.FMT_HWIO:
+        w = np.ascontiguousarray(w.transpose(2, 3, 1, 0))
+    mine = oracle.forward(oracle_shape(oracle, d, fmts), x, w)
+    ref = reflib.forward(d, x, w, fmts=fmts)
+    assert ref["bcast_applicable"]
+    for key in KEYS:
+        assert same_bytes(mine[key], ref[key]), key
+    assert mine["dst"].shape == ref["dst"].shape

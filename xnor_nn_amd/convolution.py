@@ -71,6 +71,9 @@ class Convolution:
         handle = getattr(stream, "cuda_stream", stream)
         self._check(self.lib.xnor_nn_hip_set_stream(C.byref(self.desc), handle))
 
+    def set_stage_fusion(self, on):
+        self._check(self.lib.xnor_nn_hip_set_stage_fusion(C.byref(self.desc), int(bool(on))))
+
     def synchronize(self):
         self._check(self.lib.xnor_nn_hip_synchronize(C.byref(self.desc)))
 

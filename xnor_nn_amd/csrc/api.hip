@@ -7,7 +7,11 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <iterator>
+#include <mutex>
 #include <new>
+#include <unordered_map>
+#include <utility>
 #include <vector>
 
 #include "plan.hpp"
@@ -55,16 +59,97 @@ xnor_nn_status_t unimplemented_stage(const xnor_nn_convolution_t *, xnor_nn_reso
     return xnor_nn_unimplemented;
 }
 
-// Runs the box filter that calculate_k left to the convolution (see State::k_owed_a).
-xnor_nn_status_t settle_k(State *st) {
-    if (st->k_owed_a == nullptr) return xnor_nn_success;
-    const float *a = st->k_owed_a;
-    float *k = st->k_owed_k;
-    st->k_owed_a = nullptr;
-    st->k_owed_k = nullptr;
+// ---- what one stage hands to the next ---------------------------------------------------
+// The executors are stateless apart from the launch plan behind c->state, like the
+// reference's (reference src/bcast_convolution.hpp:77-93): what a stage hands to a later one
+// is recorded against the device buffers of the caller's resource table, so two threads
+// that share a descriptor and bring a table each do not see each other's hand-overs.
+//   ready: binarize_data has also left mean|x| of this input in this `a` plane; the
+//          calculate_k that follows it immediately on the same buffers skips its own pass
+//          over the input.  Any other executor on the table withdraws the offer.
+//   owed:  calculate_k has mean|x| in `a` and has not run the box filter, because the
+//          matrix-core convolution sums K from mean|x| on the fly and stores it to this K
+//          plane.  Whatever else needs the K plane, or is about to overwrite that mean|x|,
+//          runs the box filter first.
+// Entries die with the buffers (xnor_nn_free_resources) and with the descriptor.
+struct Ready { const State *st; const void *src; };
+struct Owed { const State *st; const float *a; };
+std::mutex handover_mu;
+std::unordered_map<const void *, Ready> ready_by_a;
+std::unordered_map<const void *, Owed> owed_by_k;
+
+bool fusion_on(const State *st) {
+    return st->fuse_stages && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr;
+}
+
+void withdraw_ready(const void *a) {
+    if (a == nullptr) return;
+    std::lock_guard<std::mutex> lock(handover_mu);
+    ready_by_a.erase(a);
+}
+
+// Takes the entry for k out of the table; false when there is none.
+bool take_owed(const void *k, Owed *out) {
+    std::lock_guard<std::mutex> lock(handover_mu);
+    auto it = owed_by_k.find(k);
+    if (it == owed_by_k.end()) return false;
+    *out = it->second;
+    owed_by_k.erase(it);
+    return true;
+}
+
+xnor_nn_status_t run_box_filter(const State *st, const Owed &o, float *k) {
     if (st->verbose) printf("xnor_nn exec (deferred calculate_k): box_filter_kernel\n");
-    return launch_box_filter(st->g, a, k, st->stream) == hipSuccess ? xnor_nn_success
-                                                                    : xnor_nn_error_memory;
+    return launch_box_filter(o.st->g, o.a, k, st->stream) == hipSuccess ? xnor_nn_success
+                                                                        : xnor_nn_error_memory;
+}
+
+// Runs the box filter owed to the K plane k, if any.
+xnor_nn_status_t settle_k(const State *st, float *k) {
+    Owed o;
+    if (!take_owed(k, &o)) return xnor_nn_success;
+    return run_box_filter(st, o, k);
+}
+
+// Runs every box filter that still has to read the mean|x| plane a (about to be overwritten),
+// except the one owed to skip_k, which is dropped: its K plane is about to be recomputed.
+xnor_nn_status_t settle_readers_of(const State *st, const float *a, const void *skip_k) {
+    std::vector<std::pair<float *, Owed>> todo;
+    {
+        std::lock_guard<std::mutex> lock(handover_mu);
+        if (skip_k) owed_by_k.erase(skip_k);
+        for (auto it = owed_by_k.begin(); it != owed_by_k.end();) {
+            if (it->second.a == a) {
+                todo.emplace_back(static_cast<float *>(const_cast<void *>(it->first)),
+                        it->second);
+                it = owed_by_k.erase(it);
+            } else {
+                ++it;
+            }
+        }
+    }
+    for (auto &t : todo) {
+        const xnor_nn_status_t rc = run_box_filter(st, t.second, t.first);
+        if (rc != xnor_nn_success) return rc;
+    }
+    return xnor_nn_success;
+}
+
+void forget_buffers(const void *a, const void *k) {
+    std::lock_guard<std::mutex> lock(handover_mu);
+    if (a) ready_by_a.erase(a);
+    if (k) owed_by_k.erase(k);
+    if (a)
+        for (auto it = owed_by_k.begin(); it != owed_by_k.end();)
+            it = it->second.a == a ? owed_by_k.erase(it) : std::next(it);
+}
+
+void forget_descriptor(const State *st) {
+    std::lock_guard<std::mutex> lock(handover_mu);
+    for (auto it = ready_by_a.begin(); it != ready_by_a.end();)
+        it = it->second.st == st ? ready_by_a.erase(it) : std::next(it);
+    for (auto it = owed_by_k.begin(); it != owed_by_k.end();)
+        it = it->second.st == st ? owed_by_k.erase(it) : std::next(it);
 }
 
 // ---- stage 1 --------------------------------------------------------------------------
@@ -76,13 +161,15 @@ xnor_nn_status_t exec_binarize_data(const xnor_nn_convolution_t *c, xnor_nn_reso
         return xnor_nn_error_invalid_input;
     if (!is_data_format(c->src_format)) return xnor_nn_unimplemented;
     State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
     const void *x = nullptr;
     xnor_nn_status_t rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
             src_elems(st->g) * sizeof(float), &x);
     if (rc != xnor_nn_success) return rc;
     float *a = static_cast<float *>(res[xnor_nn_resource_a]); // optional by-product
-    if (a != nullptr && a == st->k_owed_a) { // about to overwrite the mean|x| a K is owed from
-        rc = settle_k(st);
+    if (a != nullptr) { // about to overwrite the mean|x| a K may be owed from
+        withdraw_ready(a);
+        rc = settle_readers_of(st, a, nullptr);
         if (rc != xnor_nn_success) return rc;
     }
     if (st->verbose) printf("xnor_nn exec binarize_data: %s\n", binarize_kernel_name(st->g));
@@ -90,8 +177,10 @@ xnor_nn_status_t exec_binarize_data(const xnor_nn_convolution_t *c, xnor_nn_reso
                 static_cast<uint32_t *>(res[xnor_nn_resource_bin_src]), a, st->stream)
             != hipSuccess)
         return xnor_nn_error_memory;
-    st->a_ready_src = a ? res[xnor_nn_resource_user_src] : nullptr;
-    st->a_ready_buf = a;
+    if (a != nullptr && fusion_on(st)) {
+        std::lock_guard<std::mutex> lock(handover_mu);
+        ready_by_a[a] = Ready{st, res[xnor_nn_resource_user_src]};
+    }
     return xnor_nn_success;
 }
 
@@ -105,15 +194,28 @@ xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resour
         return xnor_nn_error_invalid_input;
     if (!is_data_format(c->src_format)) return xnor_nn_unimplemented;
     State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
     float *a = static_cast<float *>(res[xnor_nn_resource_a]);
-    const bool a_ready = st->a_ready_src == res[xnor_nn_resource_user_src]
-        && st->a_ready_buf == a && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr;
-    st->a_ready_src = st->a_ready_buf = nullptr; // one-shot
-    xnor_nn_status_t owed = settle_k(st); // an earlier, still deferred K (other buffers)
-    if (owed != xnor_nn_success) return owed;
+    float *k = static_cast<float *>(res[xnor_nn_resource_k]);
+    const bool fuse = fusion_on(st);
+    bool a_ready = false;
+    {
+        std::lock_guard<std::mutex> lock(handover_mu);
+        auto it = ready_by_a.find(a);
+        if (it != ready_by_a.end()) { // one-shot
+            a_ready = fuse && it->second.st == st
+                && it->second.src == res[xnor_nn_resource_user_src];
+            ready_by_a.erase(it);
+        }
+    }
+    xnor_nn_status_t rc;
     if (!a_ready) {
+        // mean|x| is about to be overwritten: box filters that still read it run first (the
+        // one owed to this K plane is dropped, the plane is recomputed below)
+        rc = settle_readers_of(st, a, k);
+        if (rc != xnor_nn_success) return rc;
         const void *x = nullptr;
-        xnor_nn_status_t rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
+        rc = stage_in(st, &st->stage_src, res[xnor_nn_resource_user_src],
                 src_elems(st->g) * sizeof(float), &x);
         if (rc != xnor_nn_success) return rc;
         if (launch_mean_abs(st->g, static_cast<const float *>(x), a, st->stream) != hipSuccess)
@@ -121,19 +223,21 @@ xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resour
     }
     // The matrix-core convolution sums K from mean|x| itself, which saves this launch; the
     // K plane is then written by the forward executor (or by whatever needs it earlier).
-    if (st->g.use_mfma && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr) {
+    if (st->g.use_mfma && fuse) {
         if (st->verbose)
             printf("xnor_nn exec calculate_k: %sbox filter deferred to the convolution\n",
                     a_ready ? "" : "mean_abs, ");
-        st->k_owed_a = a;
-        st->k_owed_k = static_cast<float *>(res[xnor_nn_resource_k]);
+        std::lock_guard<std::mutex> lock(handover_mu);
+        owed_by_k[k] = Owed{st, a};
         return xnor_nn_success;
+    }
+    {
+        std::lock_guard<std::mutex> lock(handover_mu);
+        owed_by_k.erase(k); // superseded by the filter below
     }
     if (st->verbose)
         printf("xnor_nn exec calculate_k: %sbox_filter_kernel\n", a_ready ? "" : "mean_abs + ");
-    if (launch_box_filter(st->g, a, static_cast<float *>(res[xnor_nn_resource_k]), st->stream)
-            != hipSuccess)
-        return xnor_nn_error_memory;
+    if (launch_box_filter(st->g, a, k, st->stream) != hipSuccess) return xnor_nn_error_memory;
     return xnor_nn_success;
 }
 
@@ -148,6 +252,8 @@ xnor_nn_status_t exec_binarize_weights(const xnor_nn_convolution_t *c,
         return xnor_nn_error_invalid_input;
     if (!is_weights_format(c->weights_format)) return xnor_nn_unimplemented;
     State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    withdraw_ready(res[xnor_nn_resource_a]);
     const void *w = nullptr;
     xnor_nn_status_t rc = stage_in(st, &st->stage_weights, res[xnor_nn_resource_user_weights],
             weights_elems(st->g) * sizeof(float), &w);
@@ -171,6 +277,8 @@ xnor_nn_status_t exec_binarize_weights(const xnor_nn_convolution_t *c,
 xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resources_t res,
         void *user_out, bool raw) {
     State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    withdraw_ready(res[xnor_nn_resource_a]);
     const size_t bytes = dst_elems(st->g) * 4;
     void *out = user_out;
     const bool direct = on_device(user_out);
@@ -181,31 +289,31 @@ xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resourc
     }
     const uint32_t *xbits = static_cast<const uint32_t *>(res[xnor_nn_resource_bin_src]);
     const float *alpha = static_cast<const float *>(res[xnor_nn_resource_alpha]);
-    const float *k = static_cast<const float *>(res[xnor_nn_resource_k]);
+    float *k = static_cast<float *>(res[xnor_nn_resource_k]);
     const int32_t *opc = static_cast<const int32_t *>(res[xnor_nn_resource_operations_count]);
     float *dst = raw ? nullptr : static_cast<float *>(out);
     int32_t *popc = raw ? static_cast<int32_t *>(out) : nullptr;
     hipError_t err;
+    // a K owed to exactly this K plane is computed inside the matrix-core kernel; the raw
+    // accumulators need no K at all
+    const float *a = nullptr;
+    Owed o;
+    if (!raw && take_owed(k, &o)) {
+        if (st->g.use_mfma && o.st == st) {
+            a = o.a;
+        } else {
+            const xnor_nn_status_t rc = run_box_filter(st, o, k);
+            if (rc != xnor_nn_success) return rc;
+        }
+    }
     if (st->g.use_mfma) {
         const uint32_t *wfrag = reinterpret_cast<const uint32_t *>(
                 static_cast<const char *>(res[xnor_nn_resource_bin_weights]) + st->g.wfrag_offset);
-        // a K owed for exactly this K buffer is computed inside the kernel
-        const float *a = nullptr;
-        if (!raw && st->k_owed_a != nullptr) {
-            if (st->k_owed_k == k) {
-                a = st->k_owed_a;
-                st->k_owed_a = nullptr;
-                st->k_owed_k = nullptr;
-            } else {
-                xnor_nn_status_t rc = settle_k(st);
-                if (rc != xnor_nn_success) return rc;
-            }
-        }
         if (st->verbose)
             printf("xnor_nn exec forward: %s%s\n", convolution_kernel_name(st->g),
                     a ? " (with the box filter of calculate_k)" : "");
-        err = launch_convolution_mfma(st->g, xbits, wfrag, alpha, k, opc, dst, popc, a,
-                const_cast<float *>(k), st->stream);
+        err = launch_convolution_mfma(st->g, xbits, wfrag, alpha, k, dst, popc, a, k,
+                st->stream);
     } else {
         if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
         err = launch_convolution(st->g, xbits,
@@ -353,9 +461,11 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
 void xnor_nn_destroy_convolution(xnor_nn_convolution_t *c) {
     if (c == nullptr || c->state == nullptr) return;
     State *st = state_of(c);
+    forget_descriptor(st);
     if (st->stage_src) (void)hipFree(st->stage_src);
     if (st->stage_weights) (void)hipFree(st->stage_weights);
     if (st->stage_dst) (void)hipFree(st->stage_dst);
+    if (st->float_parts) (void)hipFree(st->float_parts);
     delete st;
     c->state = nullptr;
 }
@@ -377,38 +487,71 @@ xnor_nn_status_t xnor_nn_allocate_resources(const xnor_nn_convolution_t *c,
 }
 
 void xnor_nn_free_resources(xnor_nn_resources_t res) {
+    // nothing may be handed over through buffers that are about to go
+    forget_buffers(res[xnor_nn_resource_a], res[xnor_nn_resource_k]);
     for (int i = xnor_nn_resource_internal; i < xnor_nn_resource_number; i++) {
         if (res[i]) (void)hipFree(res[i]);
         res[i] = nullptr;
     }
 }
 
+// Replaces reference src/binarize_weights_float.cpp:3-25.  Host buffers are staged through
+// device copies and the call returns when `to` is written; with both buffers on the device
+// it only enqueues two kernels on the descriptor's stream, like the executors.
 void xnor_nn_binarize_weights_float(const xnor_nn_convolution_t *c,
         const float *from, float *to) {
     const size_t n = (size_t)c->oc * c->ic * c->kh * c->kw;
     const size_t bytes = n * sizeof(float);
-    hipStream_t s = c->state ? state_of(c)->stream : nullptr;
+    State *st = c->state ? state_of(c) : nullptr;
+    hipStream_t s = st ? st->stream : nullptr;
     const bool from_dev = on_device(from), to_dev = on_device(to);
-    float *dfrom = nullptr, *dto = nullptr, *scratch = nullptr;
-    bool ok = hipMalloc((void **)&scratch, 256 * sizeof(float)) == hipSuccess;
+    float *dfrom = nullptr, *dto = nullptr, *own_parts = nullptr, *parts = nullptr;
+    bool ok = true;
+    std::unique_lock<std::mutex> call;
+    if (st) { // the partial sums live with the descriptor
+        call = std::unique_lock<std::mutex>(st->mu);
+        if (!st->float_parts)
+            ok = hipMalloc((void **)&st->float_parts, weights_float_parts() * sizeof(float))
+                == hipSuccess;
+        parts = st->float_parts;
+    } else {
+        ok = hipMalloc((void **)&own_parts, weights_float_parts() * sizeof(float)) == hipSuccess;
+        parts = own_parts;
+    }
     if (ok && !from_dev) ok = hipMalloc((void **)&dfrom, bytes) == hipSuccess
-        && hipMemcpy(dfrom, from, bytes, hipMemcpyHostToDevice) == hipSuccess;
+        && hipMemcpyAsync(dfrom, from, bytes, hipMemcpyHostToDevice, s) == hipSuccess
+        && hipStreamSynchronize(s) == hipSuccess;
     if (ok && !to_dev) ok = hipMalloc((void **)&dto, bytes) == hipSuccess;
-    if (ok) ok = launch_weights_float(from_dev ? from : dfrom, to_dev ? to : dto, n, scratch, s)
+    if (ok) ok = launch_weights_float(from_dev ? from : dfrom, to_dev ? to : dto, n, parts, s)
         == hipSuccess;
     if (ok && !to_dev) ok = hipMemcpyAsync(to, dto, bytes, hipMemcpyDeviceToHost, s) == hipSuccess;
-    if (hipStreamSynchronize(s) != hipSuccess) ok = false;
-    if (!ok) fprintf(stderr, "xnor_nn_binarize_weights_float: HIP failure, output not written\n");
+    if (dfrom || dto || own_parts || !ok) { // something of this call's has to outlive the kernels
+        if (hipStreamSynchronize(s) != hipSuccess) ok = false;
+    }
+    if (!ok) {
+        (void)hipGetLastError();
+        fprintf(stderr, "xnor_nn_binarize_weights_float: HIP failure, output not written\n");
+    }
     if (dfrom) (void)hipFree(dfrom);
     if (dto) (void)hipFree(dto);
-    if (scratch) (void)hipFree(scratch);
+    if (own_parts) (void)hipFree(own_parts);
 }
 
 // ---- include/xnor_nn_hip.h --------------------------------------------------------------
 
 xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *stream) {
     if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
-    state_of(c)->stream = static_cast<hipStream_t>(stream);
+    State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    st->stream = static_cast<hipStream_t>(stream);
+    return xnor_nn_success;
+}
+
+xnor_nn_status_t xnor_nn_hip_set_stage_fusion(const xnor_nn_convolution_t *c, int on) {
+    if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
+    State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    st->fuse_stages = on != 0;
     return xnor_nn_success;
 }
 
@@ -485,7 +628,9 @@ xnor_nn_status_t xnor_nn_hip_export_floats(const xnor_nn_convolution_t *c,
         return xnor_nn_error_invalid_input;
     if (!res[slot] || dst_bytes != c->resource_size[slot]) return xnor_nn_error_invalid_input;
     if (slot == xnor_nn_resource_k) { // a deferred box filter has to run before K is read
-        xnor_nn_status_t rc = settle_k(state_of(c));
+        State *st = state_of(c);
+        std::lock_guard<std::mutex> call(st->mu);
+        xnor_nn_status_t rc = settle_k(st, static_cast<float *>(res[slot]));
         if (rc != xnor_nn_success) return rc;
     }
     return to_host(c, res[slot], dst, dst_bytes);

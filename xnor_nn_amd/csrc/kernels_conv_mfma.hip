@@ -189,7 +189,7 @@ template <int KS, int PS, bool RAW, bool PAIR, bool DEEP>
 __global__ __launch_bounds__(256, 2)
 void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
-        const int32_t *__restrict__ opc, float *__restrict__ dst, int32_t *__restrict__ popc,
+        float *__restrict__ dst, int32_t *__restrict__ popc,
         const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
         const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
         float *__restrict__ k_out, const float inv_khw, const int ic_parts,
@@ -585,11 +585,18 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         // are awaited here, and both register sets are named as inputs after the wait: a
         // register that is dead after the loop would otherwise be handed to the epilogue's
         // address arithmetic while its load is still on the way.
+        // The same holds for the pixel fragments: the last step has started LDS reads for a
+        // step that does not exist.
         wait_all_after<PS>(acc);
         static_for<HS>([&](auto step) {
             constexpr int hs = decltype(step)::value;
             const v4i a0 = wa[hs][0], a1 = wa[hs][1], c0 = wb[hs][0], c1 = wb[hs][1];
             asm volatile("" : : "v"(a0), "v"(a1), "v"(c0), "v"(c1));
+        });
+        static_for<PS>([&](auto block) {
+            constexpr int ps = decltype(block)::value;
+            const v4i p0 = b0[ps], p1 = b1[ps];
+            asm volatile("" : : "v"(p0), "v"(p1));
         });
     }
 
@@ -612,10 +619,13 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const bool nchw = RAW || g.dst_fmt == xnor_nn_data_format_nchw;
     const uint32_t fstep = nchw ? (uint32_t)g.ohw * 4u : 4u; // bytes from a filter to the next
     int n[PS];
+    const uint32_t kh_bits = 0xFFFFFFFFu >> (32 - g.kh), kw_bits = 0xFFFFFFFFu >> (32 - g.kw);
     uint32_t off1[PS]; // one block: lanes 0..31 filter f, lanes 32..63 filter f + 4
 #pragma unroll
     for (int ps = 0; ps < PS; ps++) {
-        n[ps] = RAW ? opc[rem[ps]] : 0;
+        // operation count of the pixel (reference src/bcast_binarize_weights.cpp:126-142):
+        // channels times the taps inside the image, from the same masks the main loop used
+        n[ps] = RAW ? g.ic * __popc(rowmask[ps] & kh_bits) * __popc(colmask[ps] & kw_bits) : 0;
         const uint32_t at = nchw ? (img[ps] * (uint32_t)g.oc * (uint32_t)g.ohw + rem[ps]) * 4u
                                  : pix[ps] * (uint32_t)g.oc * 4u;
         off1[ps] = live[ps] ? at + (uint32_t)lane_hi * 4u * fstep : DROP;
@@ -909,7 +919,7 @@ int pick_ps(const Geometry &g) {
 
 template <int KS, int PS, bool PAIR, bool DEEP = false>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
-        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
     const int chunks = (g.oc + NT - 1) / NT;
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
@@ -938,12 +948,12 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     }
     if (popc)
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
-                xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
                 g.mfma_wbytes);
     else
         hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>), grid, block, lds, s,
-                xbits, wf, alpha, k, opc, dst, popc, g, rows, chunks, units, per_xcd,
+                xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
                 g.mfma_wbytes);
     return hipGetLastError();
@@ -951,25 +961,30 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
 
 template <int KS>
 hipError_t launch_mfma_deep(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
-        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
     switch (g.mfma_ps) {
-    case 1: return launch_mfma<KS, 1, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma<KS, 2, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma<KS, 3, false, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma<KS, 1, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma<KS, 2, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma<KS, 3, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }
 
 template <int KS, bool PAIR = false>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
-        const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
+        const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s) {
     switch (g.mfma_ps) {
-    case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma<KS, 3, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 4: return launch_mfma<KS, 4, PAIR>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma<KS, 3, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 4:
+        // four pixel blocks with 16 steps per tap, or with tap pairing over five words, do not
+        // fit the register file (tile_fits_registers) and are not compiled
+        if constexpr (KS < 16 && !(PAIR && KS >= 5))
+            return launch_mfma<KS, 4, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+        break;
     }
     return hipErrorInvalidValue;
 }
@@ -1031,30 +1046,30 @@ const char *mfma_kernel_name(const Geometry &g) {
 }
 
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
-        const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
+        const uint32_t *wfrag, const float *alpha, const float *k,
         float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s) {
     if (g.mfma_pair) {
         switch (g.xw) {
-        case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-        case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-        case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+        case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+        case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+        case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
         }
         return hipErrorInvalidValue;
     }
     if (g.mfma_parts > 1) {
         if (g.mfma_steps == 12)
-            return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-        return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+            return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+        return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
     }
     switch (g.mfma_steps) {
-    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 12: return launch_mfma_ps<12>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
-    case 16: return launch_mfma_ps<16>(g, xbits, wfrag, alpha, k, opc, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 12: return launch_mfma_ps<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 16: return launch_mfma_ps<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
     }
     return hipErrorInvalidValue;
 }

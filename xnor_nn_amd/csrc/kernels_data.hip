@@ -129,12 +129,14 @@ void binarize_tile(const float *__restrict__ x, uint32_t *__restrict__ bits,
                 t[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
                         src, lane_off, (uint32_t)(c0 + i) * plane_bytes, 0));
         } else {
+            // last, ragged slice: a channel past the end gets an offset outside the buffer and
+            // reads +0 (no branch per load); its bit is masked out of the word below and |+0|
+            // leaves the running sum as it is
 #pragma unroll
             for (int i = 0; i < 32; i++)
-                t[i] = (c0 + i < g.ic)
-                    ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                              src, lane_off, (uint32_t)(c0 + i) * plane_bytes, 0))
-                    : 0.f;
+                t[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        src, c0 + i < g.ic ? lane_off : 0xFFFFFFF0u,
+                        c0 + i < g.ic ? (uint32_t)(c0 + i) * plane_bytes : 0u, 0));
         }
     };
 
@@ -362,10 +364,13 @@ bool nhwc_by_lane(const Geometry &g) {
 
 } // namespace
 
-// The tiled kernel addresses the input with 32-bit byte offsets.
+// The tiled kernel addresses the input with 32-bit byte offsets and stages the packed words
+// of a tile in LDS (64 KB at most: up to 8160 channels); deeper or larger inputs run the
+// generic kernel.
 static bool tiled_nchw(const Geometry &g) {
     return g.src_fmt == xnor_nn_data_format_nchw
-        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull;
+        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull
+        && sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw) <= 64 * 1024;
 }
 
 // The NHWC kernel reads 16 bytes per load at 32-bit byte offsets.

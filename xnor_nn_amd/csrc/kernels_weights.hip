@@ -3,7 +3,15 @@
 // (reference src/bcast_binarize_weights.cpp:54-142), plus the float sign(w)*mean(w)
 // helper (reference src/binarize_weights_float.cpp:3-25).  None of this is on the
 // per-forward path, so the kernels favour exact reference order over speed.
+#include <mutex>
+
 #include "plan.hpp"
+
+// Partial sums for callers that may not allocate (xnor_nn_hip_binarize_weights_float_noalloc):
+// 256 floats per GPU for as long as the process lives.  In host code the name is only a
+// handle; the device address comes from hipGetSymbolAddress, once per device
+// (weights_float_scratch below), and kernels get that address as an argument.
+static __device__ __align__(256) float scratch[256];
 
 namespace xnor_hip {
 
@@ -197,29 +205,50 @@ void op_count_kernel(int32_t *__restrict__ opc, const Geometry g) {
     opc[p] = taps * g.ic;
 }
 
-// Deterministic two-level sum for the float-weights helper: 256 partial sums, each over a
-// contiguous slice in index order, then a serial sum of the partials.
-constexpr int PARTS = 256;
+// Deterministic two-level sum for the float-weights helper (reference
+// src/binarize_weights_float.cpp:14-20 adds every weight into one float; its OpenMP loop
+// has no reduction clause, so only its one-thread result is defined, and a sum in another
+// fixed order is within rounding of it).  Level 1: workgroup p of PARTS sums the contiguous
+// slice p, thread t taking elements t, t + 256, ... of it (coalesced) and the 256 thread
+// sums meeting in a fixed tree.  Level 2: every workgroup of the second kernel adds the PARTS
+// partial sums in the same fixed tree, so all of them multiply by the same mean.
+constexpr int PARTS = 256; // also the length of `scratch` above
 
-__global__ __launch_bounds__(PARTS)
+__device__ __forceinline__ float tree_sum_256(float v, float *lds) {
+    const int t = threadIdx.x;
+    lds[t] = v;
+    __syncthreads();
+#pragma unroll
+    for (int half = 128; half >= 1; half >>= 1) {
+        if (t < half) lds[t] = __fadd_rn(lds[t], lds[t + half]);
+        __syncthreads();
+    }
+    return lds[0];
+}
+
+__global__ __launch_bounds__(256)
 void partial_sum_kernel(const float *__restrict__ from, float *__restrict__ parts,
         const size_t n) {
+    __shared__ float lds[256];
     const size_t per = (n + PARTS - 1) / PARTS;
-    const size_t lo = threadIdx.x * per;
+    const size_t lo = (size_t)blockIdx.x * per;
     const size_t hi = lo + per < n ? lo + per : n;
     float acc = 0.f;
-    for (size_t i = lo; i < hi; i++) acc += from[i];
-    parts[threadIdx.x] = acc;
+    for (size_t i = lo + threadIdx.x; i < hi; i += 256) acc = __fadd_rn(acc, from[i]);
+    const float sum = tree_sum_256(acc, lds);
+    if (threadIdx.x == 0) parts[blockIdx.x] = sum;
 }
 
 __global__ __launch_bounds__(256)
 void sign_times_mean_kernel(const float *__restrict__ from, float *__restrict__ to,
         const float *__restrict__ parts, const size_t n, const float inv_n) {
-    float sum = 0.f;
-    for (int i = 0; i < PARTS; i++) sum += parts[i];
-    const float mean = sum * inv_n;
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) to[i] = (from[i] >= 0.f ? 1.f : -1.f) * mean;
+    __shared__ float lds[256];
+    const float mean = __fmul_rn(tree_sum_256(parts[threadIdx.x], lds), inv_n);
+    // four consecutive elements per thread
+    const size_t i0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (i0 + u < n) to[i0 + u] = from[i0 + u] >= 0.f ? mean : -mean;
 }
 
 } // namespace
@@ -242,13 +271,37 @@ hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *
     return hipGetLastError();
 }
 
-// scratch: PARTS floats of device memory.
-hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
+int weights_float_parts() { return PARTS; }
+
+// parts: PARTS floats of device memory.
+hipError_t launch_weights_float(const float *from, float *to, size_t n, float *parts,
         hipStream_t s) {
-    hipLaunchKernelGGL(partial_sum_kernel, dim3(1), dim3(PARTS), 0, s, from, scratch, n);
-    hipLaunchKernelGGL(sign_times_mean_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256),
-            0, s, from, to, scratch, n, 1.f / (float)n);
+    hipLaunchKernelGGL(partial_sum_kernel, dim3(PARTS), dim3(256), 0, s, from, parts, n);
+    hipLaunchKernelGGL(sign_times_mean_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256),
+            0, s, from, to, parts, n, 1.f / (float)n);
     return hipGetLastError();
+}
+
+// Device address of this GPU's copy of `scratch`, looked up on the first call on a device
+// (with that device current) and kept.
+hipError_t weights_float_scratch(float **out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static float *addr[MAX_DEVICES];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (addr[dev] == nullptr) {
+        float *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return hipSuccess;
 }
 
 } // namespace xnor_hip

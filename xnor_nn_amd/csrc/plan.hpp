@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "xnor_nn.h"
 
 namespace xnor_hip {
@@ -71,19 +73,19 @@ struct Geometry {
 struct State {
     Geometry g;
     hipStream_t stream = nullptr;
+    // Held for the length of every executor call: two host threads may share one descriptor
+    // (each with a resource table of its own), and the staging buffers below, the stream and
+    // the order in which a call's launches and copies are enqueued belong to one call at a
+    // time.
+    std::mutex mu;
     // staging buffers for host-side user tensors (allocated on first use)
     void *stage_src = nullptr, *stage_weights = nullptr, *stage_dst = nullptr;
-    // One-shot hand-over from binarize_data to calculate_k: binarize_data reads the
-    // input anyway and also leaves mean|x| in res[a]; calculate_k may then skip its own
-    // pass over the input when it is called next with the same src and a buffers.
-    const void *a_ready_src = nullptr;
-    const void *a_ready_buf = nullptr;
-    // K owed: calculate_k has mean|x| in k_owed_a and has not run the box filter, because
-    // the matrix-core convolution computes K from mean|x| on the fly (and stores it to
-    // k_owed_k).  Anything else that needs the K plane, or that is about to overwrite
-    // mean|x|, runs the box filter first (settle_k in api.hip).
-    const float *k_owed_a = nullptr;
-    float *k_owed_k = nullptr;
+    // partial sums of xnor_nn_binarize_weights_float (allocated on first use)
+    float *float_parts = nullptr;
+    // Stage fusion (xnor_nn_hip_set_stage_fusion): binarize_data hands mean|x| to the
+    // calculate_k that follows it, and calculate_k leaves its box filter to the matrix-core
+    // convolution.  What is handed over is recorded per resource table, not here (api.hip).
+    bool fuse_stages = true;
     bool verbose = false;
 };
 
@@ -101,8 +103,13 @@ hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *
 hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wbits, const float *alpha, const float *k, const int32_t *opc,
         float *dst, int32_t *popc_or_null, hipStream_t s);
-hipError_t launch_weights_float(const float *from, float *to, size_t n, float *scratch,
+// sign(w) * mean(w); parts: weights_float_parts() floats of device memory for partial sums
+int weights_float_parts();
+hipError_t launch_weights_float(const float *from, float *to, size_t n, float *parts,
         hipStream_t s);
+// device address of the library's own partial-sum array on the current GPU (static device
+// memory: nothing is allocated)
+hipError_t weights_float_scratch(float **out);
 // Decides whether the matrix-core kernel takes the problem and fills use_mfma, mfma_ps and
 // the mfma_* fields (everything the launch needs, so that a forward call computes nothing).
 void mfma_plan(Geometry &g);
@@ -113,7 +120,7 @@ hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *
 // With a_or_null set, the kernel ignores k, computes the K plane itself from mean|x| (the
 // box filter of stage 2) and also stores it to k_out.
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
-        const uint32_t *wfrag, const float *alpha, const float *k, const int32_t *opc,
+        const uint32_t *wfrag, const float *alpha, const float *k,
         float *dst, int32_t *popc_or_null, const float *a_or_null, float *k_out,
         hipStream_t s);
 const char *convolution_kernel_name(const Geometry &g);

@@ -43,7 +43,8 @@ class XnorConv2d(torch.nn.Module):
         (kh, kw), (sh, sw), (ph, pw) = self.kernel_size, self.stride, self.padding
         self._conv = Convolution(capi.ALGORITHM_BCAST, capi.FMT_NCHW, capi.FMT_OIHW,
                                  capi.FMT_NCHW, mb, self.out_channels, ic, ih, iw,
-                                 kh, kw, sh, sw, ph, pw, self.weight.data)
+                                 kh, kw, sh, sw, ph, pw, self.weight.data,
+                                 stream=torch.cuda.current_stream(x.device))
         self._shape = tuple(x.shape)
         self._weights_changed = False
 
@@ -55,14 +56,17 @@ class XnorConv2d(torch.nn.Module):
         if self.weight.device != x.device:
             raise ValueError("weight and input live on different devices")
         x = x.contiguous()
+        # every kernel of this call, the weight stage included, goes to torch's current stream:
+        # that orders it behind the writes to `weight` and `x` already enqueued there
         if self._conv is None or self._shape != tuple(x.shape):
             self._build(x)
-        elif self._weights_changed:
-            self._conv.change_weights(self.weight.data)
-            self._weights_changed = False
+        else:
+            self._conv.set_stream(torch.cuda.current_stream(x.device))
+            if self._weights_changed:
+                self._conv.change_weights(self.weight.data)
+                self._weights_changed = False
         d = self._conv.desc
         y = torch.empty((d.mb, d.oc, d.oh, d.ow), dtype=torch.float32, device=x.device)
-        self._conv.set_stream(torch.cuda.current_stream(x.device))
         self._conv.forward(x, y)
         return y
 
@@ -73,5 +77,6 @@ class XnorConv2d(torch.nn.Module):
         if self._conv is None:
             raise RuntimeError("run a forward pass first (the descriptor is built there)")
         out = torch.empty_like(self.weight.data)
+        self._conv.set_stream(torch.cuda.current_stream(out.device))
         self._conv.binarizeWeightsFloat(self.weight.data, out)
         return out
