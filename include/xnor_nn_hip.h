@@ -95,6 +95,18 @@ xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
 int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage,
         char *buf, size_t buf_bytes);
 
+/* Kernel durations as the GPU saw them, for benchmarks: with capacity > 0 every launch of
+ * the binarize and of the convolution kernel by this descriptor's executors gets a pair of
+ * HIP events attached to its own dispatch (hipExtLaunchKernel; no extra packets on the
+ * stream), kept in a ring of `capacity` launches per stage; capacity = 0 switches timing
+ * off.  xnor_nn_hip_kernel_times waits for the stream, writes the durations (milliseconds,
+ * oldest first) of the launches of `stage` (xnor_nn_operation_binarize_data or
+ * xnor_nn_operation_convolution_forward) since the last query into ms[0..max) and returns
+ * how many it wrote, -1 on error.  The counterpart of the per-stage timers of reference
+ * test/perf/test_simple_net.cpp:60-88. */
+xnor_nn_status_t xnor_nn_hip_time_kernels(const xnor_nn_convolution_t *c, int capacity);
+int xnor_nn_hip_kernel_times(const xnor_nn_convolution_t *c, int stage, float *ms, int max);
+
 /* Compute units and peak engine clock (kHz) of the current HIP device, as the runtime
  * reports them; the figures the VALU roofline of the convolution kernel is priced with.
  * The reference's counterpart is its CPUID probe (reference src/utils/cpuid.hpp:119-168). */

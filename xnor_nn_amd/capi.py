@@ -19,6 +19,9 @@ RES_INTERNAL = 3
 # xnor_nn_tensor_format_t
 FMT_NCHW, FMT_NHWC, FMT_OIHW, FMT_HWIO = range(4)
 
+# xnor_nn_operation_t
+(OP_CONVOLUTION_FORWARD, OP_BINARIZE_WEIGHTS, OP_BINARIZE_DATA, OP_CALCULATE_K) = range(4)
+
 Resources = C.c_void_p * RES_NUMBER
 
 
@@ -69,6 +72,8 @@ HIP_SYMBOLS = {
     "xnor_nn_hip_forward_popcount": (C.c_int, [C.POINTER(ConvolutionDesc), C.POINTER(C.c_void_p), C.c_void_p]),
     "xnor_nn_hip_canonical_bici": (C.c_int, [C.POINTER(ConvolutionDesc)]),
     "xnor_nn_hip_device_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "xnor_nn_hip_time_kernels": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int]),
+    "xnor_nn_hip_kernel_times": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int, C.POINTER(C.c_float), C.c_int]),
     "xnor_nn_hip_kernel_name": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int, C.c_char_p, C.c_size_t]),
 }
 

@@ -74,6 +74,19 @@ class Convolution:
     def set_stage_fusion(self, on):
         self._check(self.lib.xnor_nn_hip_set_stage_fusion(C.byref(self.desc), int(bool(on))))
 
+    def time_kernels(self, capacity):
+        """Attach HIP events to the next launches of the binarize and convolution kernels
+        (a ring of `capacity` launches per stage; 0 switches it off)."""
+        self._check(self.lib.xnor_nn_hip_time_kernels(C.byref(self.desc), capacity))
+
+    def kernel_times(self, stage, max_launches=65536):
+        """Durations in milliseconds of the timed launches of one stage since the last call."""
+        buf = (C.c_float * max_launches)()
+        n = self.lib.xnor_nn_hip_kernel_times(C.byref(self.desc), stage, buf, max_launches)
+        if n < 0:
+            raise XnorNNError("kernel times are not available")
+        return list(buf[:n])
+
     def synchronize(self):
         self._check(self.lib.xnor_nn_hip_synchronize(C.byref(self.desc)))
 

@@ -174,7 +174,8 @@ xnor_nn_status_t exec_binarize_data(const xnor_nn_convolution_t *c, xnor_nn_reso
     }
     if (st->verbose) printf("xnor_nn exec binarize_data: %s\n", binarize_kernel_name(st->g));
     if (launch_binarize_data(st->g, static_cast<const float *>(x),
-                static_cast<uint32_t *>(res[xnor_nn_resource_bin_src]), a, st->stream)
+                static_cast<uint32_t *>(res[xnor_nn_resource_bin_src]), a, st->stream,
+                st->time_binarize.next())
             != hipSuccess)
         return xnor_nn_error_memory;
     if (a != nullptr && fusion_on(st)) {
@@ -313,12 +314,12 @@ xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resourc
             printf("xnor_nn exec forward: %s%s\n", convolution_kernel_name(st->g),
                     a ? " (with the box filter of calculate_k)" : "");
         err = launch_convolution_mfma(st->g, xbits, wfrag, alpha, k, dst, popc, a, k,
-                st->stream);
+                st->stream, st->time_convolution.next());
     } else {
         if (st->verbose) printf("xnor_nn exec forward: %s\n", convolution_kernel_name(st->g));
         err = launch_convolution(st->g, xbits,
                 static_cast<const uint32_t *>(res[xnor_nn_resource_bin_weights]), alpha, k, opc,
-                dst, popc, st->stream);
+                dst, popc, st->stream, st->time_convolution.next());
     }
     if (err != hipSuccess) return xnor_nn_error_memory;
     if (!direct) {
@@ -350,6 +351,30 @@ xnor_nn_status_t to_host(const xnor_nn_convolution_t *c, const void *dev, void *
             || hipStreamSynchronize(st->stream) != hipSuccess)
         return xnor_nn_error_memory;
     return xnor_nn_success;
+}
+
+void drop_timer(KernelTimer &t) {
+    for (KernelEvents &e : t.ring) {
+        if (e.start) (void)hipEventDestroy(e.start);
+        if (e.stop) (void)hipEventDestroy(e.stop);
+    }
+    t.ring.clear();
+    t.launches = 0;
+}
+
+bool make_timer(KernelTimer &t, int capacity) {
+    drop_timer(t);
+    for (int i = 0; i < capacity; i++) {
+        KernelEvents e;
+        if (hipEventCreate(&e.start) != hipSuccess || hipEventCreate(&e.stop) != hipSuccess) {
+            if (e.start) (void)hipEventDestroy(e.start);
+            (void)hipGetLastError();
+            drop_timer(t);
+            return false;
+        }
+        t.ring.push_back(e);
+    }
+    return true;
 }
 
 int canonical_bici(const Geometry &g) { return (g.ic * g.kh * g.kw < 32767) ? 2 : 4; }
@@ -466,6 +491,8 @@ void xnor_nn_destroy_convolution(xnor_nn_convolution_t *c) {
     if (st->stage_weights) (void)hipFree(st->stage_weights);
     if (st->stage_dst) (void)hipFree(st->stage_dst);
     if (st->float_parts) (void)hipFree(st->float_parts);
+    drop_timer(st->time_binarize);
+    drop_timer(st->time_convolution);
     delete st;
     c->state = nullptr;
 }
@@ -553,6 +580,40 @@ xnor_nn_status_t xnor_nn_hip_set_stage_fusion(const xnor_nn_convolution_t *c, in
     std::lock_guard<std::mutex> call(st->mu);
     st->fuse_stages = on != 0;
     return xnor_nn_success;
+}
+
+xnor_nn_status_t xnor_nn_hip_time_kernels(const xnor_nn_convolution_t *c, int capacity) {
+    if (!bcast_descriptor(c) || capacity < 0 || capacity > 65536)
+        return xnor_nn_error_invalid_input;
+    State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    if (hipStreamSynchronize(st->stream) != hipSuccess) return xnor_nn_error_memory;
+    if (!make_timer(st->time_binarize, capacity) || !make_timer(st->time_convolution, capacity))
+        return xnor_nn_error_memory;
+    return xnor_nn_success;
+}
+
+int xnor_nn_hip_kernel_times(const xnor_nn_convolution_t *c, int stage, float *ms, int max) {
+    if (!bcast_descriptor(c) || ms == nullptr || max < 0) return -1;
+    State *st = state_of(c);
+    std::lock_guard<std::mutex> call(st->mu);
+    KernelTimer *t = stage == xnor_nn_operation_binarize_data ? &st->time_binarize
+        : stage == xnor_nn_operation_convolution_forward ? &st->time_convolution : nullptr;
+    if (t == nullptr) return -1;
+    if (hipStreamSynchronize(st->stream) != hipSuccess) return -1;
+    const size_t have = t->launches < t->ring.size() ? t->launches : t->ring.size();
+    const size_t first = t->launches - have; // oldest launch still in the ring
+    int n = 0;
+    for (size_t i = first; i < t->launches && n < max; i++) {
+        const KernelEvents &e = t->ring[i % t->ring.size()];
+        if (hipEventElapsedTime(&ms[n], e.start, e.stop) != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;
+        }
+        n++;
+    }
+    t->launches = 0;
+    return n;
 }
 
 xnor_nn_status_t xnor_nn_hip_synchronize(const xnor_nn_convolution_t *c) {

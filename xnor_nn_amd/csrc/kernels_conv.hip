@@ -139,14 +139,14 @@ void conv_xnor_popc_kernel(const uint32_t *__restrict__ xbits,
 template <int XW, int Q>
 hipError_t launch_variant(const Geometry &g, const uint32_t *xbits, const uint32_t *wbits,
         const float *alpha, const float *k, const int32_t *opc, float *dst, int32_t *popc,
-        hipStream_t s) {
+        hipStream_t s, const KernelEvents &ev) {
     const dim3 grid((g.npix_out + 63) / 64, (g.ocb + WAVES - 1) / WAVES);
     const dim3 block(64 * WAVES);
     if (popc)
-        hipLaunchKernelGGL((conv_xnor_popc_kernel<XW, Q, true>), grid, block, 0, s, xbits,
+        launch_kernel(conv_xnor_popc_kernel<XW, Q, true>, grid, block, 0, s, ev, xbits,
                 wbits, alpha, k, opc, dst, popc, g);
     else
-        hipLaunchKernelGGL((conv_xnor_popc_kernel<XW, Q, false>), grid, block, 0, s, xbits,
+        launch_kernel(conv_xnor_popc_kernel<XW, Q, false>, grid, block, 0, s, ev, xbits,
                 wbits, alpha, k, opc, dst, popc, g);
     return hipGetLastError();
 }
@@ -170,10 +170,10 @@ const char *convolution_kernel_name(const Geometry &g) {
 
 hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wbits, const float *alpha, const float *k, const int32_t *opc,
-        float *dst, int32_t *popc, hipStream_t s) {
+        float *dst, int32_t *popc, hipStream_t s, const KernelEvents &ev) {
 #define XNOR_CASE(XW_, Q_) \
     if (g.q == Q_ && (XW_ == 0 || g.xw == XW_)) \
-        return launch_variant<XW_, Q_>(g, xbits, wbits, alpha, k, opc, dst, popc, s);
+        return launch_variant<XW_, Q_>(g, xbits, wbits, alpha, k, opc, dst, popc, s, ev);
     XNOR_CASE(3, 16)
     XNOR_CASE(8, 16)
     XNOR_CASE(12, 16)

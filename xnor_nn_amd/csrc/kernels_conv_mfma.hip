@@ -292,7 +292,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     for (int i = tid; i < ROW_BYTES / 4; i += 256) reinterpret_cast<uint32_t *>(rows)[i] = 0;
     // asked for now, put into LDS after the expansion: nothing needs it before the epilogue,
     // and the first barrier does not have to wait for it
-    const float alpha_early = chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
+    // (the raw-accumulator variant takes a table that need not hold alpha at all)
+    const float alpha_early = !RAW && chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
     if (fuse_k) { // mean|x| of the staged input pixels, plus one slot that holds zero
         if (tid < nrows) a_lds[tid] = a_early;
         if (tid == 0) a_lds[max_rows] = 0.f;
@@ -920,7 +921,7 @@ int pick_ps(const Geometry &g) {
 template <int KS, int PS, bool PAIR, bool DEEP = false>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
-        const float *a_or_null, float *k_out, hipStream_t s) {
+        const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     const int chunks = (g.oc + NT - 1) / NT;
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
     const uint32_t units = tiles * chunks, per_xcd = (units + 7) / 8;
@@ -947,12 +948,12 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         }
     }
     if (popc)
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>), grid, block, lds, s,
+        launch_kernel(conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>, grid, block, lds, s, ev,
                 xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
                 g.mfma_wbytes);
     else
-        hipLaunchKernelGGL((conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>), grid, block, lds, s,
+        launch_kernel(conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>, grid, block, lds, s, ev,
                 xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
                 g.mfma_wbytes);
@@ -962,11 +963,11 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
 template <int KS>
 hipError_t launch_mfma_deep(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
-        const float *a_or_null, float *k_out, hipStream_t s) {
+        const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     switch (g.mfma_ps) {
-    case 1: return launch_mfma<KS, 1, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma<KS, 2, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma<KS, 3, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma<KS, 1, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 2: return launch_mfma<KS, 2, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 3: return launch_mfma<KS, 3, false, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
     }
     return hipErrorInvalidValue;
 }
@@ -974,16 +975,16 @@ hipError_t launch_mfma_deep(const Geometry &g, const uint32_t *xbits, const uint
 template <int KS, bool PAIR = false>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
-        const float *a_or_null, float *k_out, hipStream_t s) {
+        const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     switch (g.mfma_ps) {
-    case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma<KS, 3, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 3: return launch_mfma<KS, 3, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
     case 4:
         // four pixel blocks with 16 steps per tap, or with tap pairing over five words, do not
         // fit the register file (tile_fits_registers) and are not compiled
         if constexpr (KS < 16 && !(PAIR && KS >= 5))
-            return launch_mfma<KS, 4, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+            return launch_mfma<KS, 4, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
         break;
     }
     return hipErrorInvalidValue;
@@ -1047,29 +1048,29 @@ const char *mfma_kernel_name(const Geometry &g) {
 
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k,
-        float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s) {
+        float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     if (g.mfma_pair) {
         switch (g.xw) {
-        case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-        case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-        case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+        case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+        case 3: return launch_mfma_ps<3, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+        case 5: return launch_mfma_ps<5, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
         }
         return hipErrorInvalidValue;
     }
     if (g.mfma_parts > 1) {
         if (g.mfma_steps == 12)
-            return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-        return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+            return launch_mfma_deep<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+        return launch_mfma_deep<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
     }
     switch (g.mfma_steps) {
-    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 12: return launch_mfma_ps<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
-    case 16: return launch_mfma_ps<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s);
+    case 1: return launch_mfma_ps<1>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 2: return launch_mfma_ps<2>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 3: return launch_mfma_ps<3>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 4: return launch_mfma_ps<4>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 6: return launch_mfma_ps<6>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 8: return launch_mfma_ps<8>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 12: return launch_mfma_ps<12>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
+    case 16: return launch_mfma_ps<16>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
     }
     return hipErrorInvalidValue;
 }

@@ -324,7 +324,8 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
 }
 
 template <bool NHWC, bool WRITE_BITS, bool WRITE_A>
-void launch_tiled(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s) {
+void launch_tiled(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s,
+        const KernelEvents &ev) {
     // At most twelve waves per workgroup, the slices split evenly over the rounds: with more
     // waves the hand-over chain of one workgroup gets long and too few workgroups are
     // resident to cover it (512 input channels: 14.1 us with 16 waves, 10.4 us with 2 x 8;
@@ -343,11 +344,11 @@ void launch_tiled(const Geometry &g, const float *x, uint32_t *bits, float *a, h
     size_t lds = sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw);
     if (NHWC) lds = ((lds + 15) & ~(size_t)15) + sizeof(float) * nw * 32 * TURN_ROW;
     if (NHWC)
-        hipLaunchKernelGGL((binarize_nhwc_tiled_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
-                dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+        launch_kernel(binarize_nhwc_tiled_kernel<WRITE_BITS, WRITE_A>, dim3(per_xcd * 8),
+                dim3(nw * TILE), lds, s, ev, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
     else
-        hipLaunchKernelGGL((binarize_nchw_kernel<WRITE_BITS, WRITE_A>), dim3(per_xcd * 8),
-                dim3(nw * TILE), lds, s, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
+        launch_kernel(binarize_nchw_kernel<WRITE_BITS, WRITE_A>, dim3(per_xcd * 8),
+                dim3(nw * TILE), lds, s, ev, x, bits, a, g, 1.f / g.ic, rounds, ntiles, per_xcd);
 }
 
 // NHWC input runs the tiled kernel unless its LDS (chain, packed words, turn-around rows) would
@@ -386,30 +387,30 @@ const char *binarize_kernel_name(const Geometry &g) {
 }
 
 hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
-        float *a_or_null, hipStream_t s) {
+        float *a_or_null, hipStream_t s, const KernelEvents &ev) {
     const float inv_ic = 1.f / g.ic;
     if (tiled_nchw(g)) {
-        if (a_or_null) launch_tiled<false, true, true>(g, x, bits, a_or_null, s);
-        else launch_tiled<false, true, false>(g, x, bits, nullptr, s);
+        if (a_or_null) launch_tiled<false, true, true>(g, x, bits, a_or_null, s, ev);
+        else launch_tiled<false, true, false>(g, x, bits, nullptr, s, ev);
     } else if (vector_nhwc(g) && !nhwc_by_lane(g)) {
-        if (a_or_null) launch_tiled<true, true, true>(g, x, bits, a_or_null, s);
-        else launch_tiled<true, true, false>(g, x, bits, nullptr, s);
+        if (a_or_null) launch_tiled<true, true, true>(g, x, bits, a_or_null, s, ev);
+        else launch_tiled<true, true, false>(g, x, bits, nullptr, s, ev);
     } else if (vector_nhwc(g)) {
         const unsigned blocks = (g.npix_in + 255) / 256;
         if (a_or_null)
-            hipLaunchKernelGGL((binarize_nhwc_kernel<true, true>), dim3(blocks), dim3(256), 0,
-                    s, x, bits, a_or_null, g, inv_ic);
+            launch_kernel(binarize_nhwc_kernel<true, true>, dim3(blocks), dim3(256), 0, s, ev,
+                    x, bits, a_or_null, g, inv_ic);
         else
-            hipLaunchKernelGGL((binarize_nhwc_kernel<true, false>), dim3(blocks), dim3(256), 0,
-                    s, x, bits, a_or_null, g, inv_ic);
+            launch_kernel(binarize_nhwc_kernel<true, false>, dim3(blocks), dim3(256), 0, s, ev,
+                    x, bits, a_or_null, g, inv_ic);
     } else {
         const unsigned blocks = (g.npix_in + 255) / 256;
         if (a_or_null)
-            hipLaunchKernelGGL((binarize_generic_kernel<true, true>), dim3(blocks),
-                    dim3(256), 0, s, x, bits, a_or_null, g, inv_ic);
+            launch_kernel(binarize_generic_kernel<true, true>, dim3(blocks), dim3(256), 0, s,
+                    ev, x, bits, a_or_null, g, inv_ic);
         else
-            hipLaunchKernelGGL((binarize_generic_kernel<true, false>), dim3(blocks),
-                    dim3(256), 0, s, x, bits, a_or_null, g, inv_ic);
+            launch_kernel(binarize_generic_kernel<true, false>, dim3(blocks), dim3(256), 0, s,
+                    ev, x, bits, a_or_null, g, inv_ic);
     }
     return hipGetLastError();
 }
@@ -417,9 +418,9 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s) {
     const float inv_ic = 1.f / g.ic;
     if (tiled_nchw(g)) {
-        launch_tiled<false, false, true>(g, x, nullptr, a, s);
+        launch_tiled<false, false, true>(g, x, nullptr, a, s, KernelEvents{});
     } else if (vector_nhwc(g) && !nhwc_by_lane(g)) {
-        launch_tiled<true, false, true>(g, x, nullptr, a, s);
+        launch_tiled<true, false, true>(g, x, nullptr, a, s, KernelEvents{});
     } else if (vector_nhwc(g)) {
         const unsigned blocks = (g.npix_in + 255) / 256;
         hipLaunchKernelGGL((binarize_nhwc_kernel<false, true>), dim3(blocks), dim3(256), 0, s,

@@ -8,9 +8,11 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <mutex>
+#include <vector>
 
 #include "xnor_nn.h"
 
@@ -70,6 +72,33 @@ struct Geometry {
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
 
+// Optional timing of one launch: when both events are set the kernel is launched with them
+// attached to its own dispatch, and their difference is the kernel's duration on the GPU (no
+// marker packets on the stream, which would cost more than a short kernel takes).
+struct KernelEvents {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+
+template <class K, class... A>
+inline void launch_kernel(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s,
+        const KernelEvents &ev, A... args) {
+    if (ev.start != nullptr && ev.stop != nullptr)
+        hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, s, ev.start, ev.stop, 0,
+                args...);
+    else
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, args...);
+}
+
+// Event pairs for xnor_nn_hip_time_kernels: one ring per timed stage.
+struct KernelTimer {
+    std::vector<KernelEvents> ring;
+    size_t launches = 0; // since timing was switched on
+    KernelEvents next() {
+        if (ring.empty()) return KernelEvents{};
+        return ring[launches++ % ring.size()];
+    }
+};
+
 struct State {
     Geometry g;
     hipStream_t stream = nullptr;
@@ -87,6 +116,7 @@ struct State {
     // convolution.  What is handed over is recorded per resource table, not here (api.hip).
     bool fuse_stages = true;
     bool verbose = false;
+    KernelTimer time_binarize, time_convolution; // empty unless timing is switched on
 };
 
 inline State *state_of(const xnor_nn_convolution_t *c) {
@@ -95,21 +125,19 @@ inline State *state_of(const xnor_nn_convolution_t *c) {
 
 // Kernel launchers (one per stage); each returns the hipError_t of the launch.
 hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bits,
-        float *a_or_null, hipStream_t s);
+        float *a_or_null, hipStream_t s, const KernelEvents &ev = KernelEvents{});
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s);
 hipError_t launch_box_filter(const Geometry &g, const float *a, float *k, hipStream_t s);
 hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *bits,
         float *alpha, int32_t *opc, hipStream_t s);
 hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wbits, const float *alpha, const float *k, const int32_t *opc,
-        float *dst, int32_t *popc_or_null, hipStream_t s);
+        float *dst, int32_t *popc_or_null, hipStream_t s,
+        const KernelEvents &ev = KernelEvents{});
 // sign(w) * mean(w); parts: weights_float_parts() floats of device memory for partial sums
 int weights_float_parts();
 hipError_t launch_weights_float(const float *from, float *to, size_t n, float *parts,
         hipStream_t s);
-// device address of the library's own partial-sum array on the current GPU (static device
-// memory: nothing is allocated)
-hipError_t weights_float_scratch(float **out);
 // Decides whether the matrix-core kernel takes the problem and fills use_mfma, mfma_ps and
 // the mfma_* fields (everything the launch needs, so that a forward call computes nothing).
 void mfma_plan(Geometry &g);
@@ -122,7 +150,7 @@ hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k,
         float *dst, int32_t *popc_or_null, const float *a_or_null, float *k_out,
-        hipStream_t s);
+        hipStream_t s, const KernelEvents &ev = KernelEvents{});
 const char *convolution_kernel_name(const Geometry &g);
 const char *binarize_kernel_name(const Geometry &g);
 
