@@ -112,6 +112,21 @@ int xnor_nn_hip_kernel_times(const xnor_nn_convolution_t *c, int stage, float *m
  * The reference's counterpart is its CPUID probe (reference src/utils/cpuid.hpp:119-168). */
 xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz);
 
+/* xnor_nn_binarize_weights_float (reference src/binarize_weights_float.cpp:3-25) for callers
+ * that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  `from` and `to`
+ * must both be device pointers to OC*IC*KH*KW floats; the call enqueues two kernels on the
+ * descriptor's stream and returns (no allocation, no free, no memset, no synchronisation),
+ * and writes the same bits as xnor_nn_binarize_weights_float.  The 256 partial sums live in
+ * a 1 KB device array that is part of the library and stays on every GPU the library has
+ * run on until the process ends.  Every call on a GPU shares that array: calls that overlap
+ * on one GPU (two streams, two threads) race on it and must be ordered by the caller.
+ * More than XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS weights, or a host pointer that is null, is
+ * refused with xnor_nn_error_invalid_input and a line on stderr. */
+#define XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS 2147483647LL /* the reference counts them in an int */
+xnor_nn_status_t xnor_nn_hip_binarize_weights_float_noalloc(const xnor_nn_convolution_t *c,
+        const float *from, float *to);
+
 #ifdef __cplusplus
 }
 #endif

@@ -72,6 +72,7 @@ HIP_SYMBOLS = {
     "xnor_nn_hip_forward_popcount": (C.c_int, [C.POINTER(ConvolutionDesc), C.POINTER(C.c_void_p), C.c_void_p]),
     "xnor_nn_hip_canonical_bici": (C.c_int, [C.POINTER(ConvolutionDesc)]),
     "xnor_nn_hip_device_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "xnor_nn_hip_binarize_weights_float_noalloc": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_void_p, C.c_void_p]),
     "xnor_nn_hip_time_kernels": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int]),
     "xnor_nn_hip_kernel_times": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int, C.POINTER(C.c_float), C.c_int]),
     "xnor_nn_hip_kernel_name": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int, C.c_char_p, C.c_size_t]),

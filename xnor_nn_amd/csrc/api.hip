@@ -566,6 +566,29 @@ void xnor_nn_binarize_weights_float(const xnor_nn_convolution_t *c,
 
 // ---- include/xnor_nn_hip.h --------------------------------------------------------------
 
+// xnor_nn_binarize_weights_float for callers that may not allocate: both buffers on the
+// device, partial sums in the library's static device array, two kernels enqueued on the
+// descriptor's stream, nothing else.
+xnor_nn_status_t xnor_nn_hip_binarize_weights_float_noalloc(const xnor_nn_convolution_t *c,
+        const float *from, float *to) {
+    if (c == nullptr || from == nullptr || to == nullptr) return xnor_nn_error_invalid_input;
+    const long long n = (long long)c->oc * c->ic * c->kh * c->kw;
+    if (c->oc <= 0 || c->ic <= 0 || c->kh <= 0 || c->kw <= 0
+            || n > XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS) {
+        fprintf(stderr, "xnor_nn_hip_binarize_weights_float_noalloc: %lld weights, the limit "
+                "is %lld\n", n, (long long)XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS);
+        return xnor_nn_error_invalid_input;
+    }
+    float *parts = nullptr;
+    if (weights_float_scratch(&parts) != hipSuccess) {
+        (void)hipGetLastError();
+        return xnor_nn_error_memory;
+    }
+    hipStream_t s = c->state ? state_of(c)->stream : nullptr;
+    return launch_weights_float(from, to, (size_t)n, parts, s) == hipSuccess
+        ? xnor_nn_success : xnor_nn_error_memory;
+}
+
 xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *stream) {
     if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
     State *st = state_of(c);

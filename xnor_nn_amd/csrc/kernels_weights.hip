@@ -7,6 +7,12 @@
 
 #include "plan.hpp"
 
+// Partial sums for callers that may not allocate (xnor_nn_hip_binarize_weights_float_noalloc):
+// 256 floats per GPU for as long as the process lives.  In host code the name is only a
+// handle; the device address comes from hipGetSymbolAddress, once per device
+// (weights_float_scratch below), and kernels get that address as an argument.
+static __device__ __align__(256) float scratch[256];
+
 namespace xnor_hip {
 
 namespace {
@@ -206,7 +212,7 @@ void op_count_kernel(int32_t *__restrict__ opc, const Geometry g) {
 // slice p, thread t taking elements t, t + 256, ... of it (coalesced) and the 256 thread
 // sums meeting in a fixed tree.  Level 2: every workgroup of the second kernel adds the PARTS
 // partial sums in the same fixed tree, so all of them multiply by the same mean.
-constexpr int PARTS = 256;
+constexpr int PARTS = 256; // also the length of `scratch` above
 
 __device__ __forceinline__ float tree_sum_256(float v, float *lds) {
     const int t = threadIdx.x;
@@ -274,6 +280,28 @@ hipError_t launch_weights_float(const float *from, float *to, size_t n, float *p
     hipLaunchKernelGGL(sign_times_mean_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256),
             0, s, from, to, parts, n, 1.f / (float)n);
     return hipGetLastError();
+}
+
+// Device address of this GPU's copy of `scratch`, looked up on the first call on a device
+// (with that device current) and kept.
+hipError_t weights_float_scratch(float **out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static float *addr[MAX_DEVICES];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (addr[dev] == nullptr) {
+        float *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return hipSuccess;
 }
 
 } // namespace xnor_hip

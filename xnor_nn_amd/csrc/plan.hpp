@@ -138,6 +138,9 @@ hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
 int weights_float_parts();
 hipError_t launch_weights_float(const float *from, float *to, size_t n, float *parts,
         hipStream_t s);
+// device address of the library's own partial-sum array on the current GPU (static device
+// memory: nothing is allocated)
+hipError_t weights_float_scratch(float **out);
 // Decides whether the matrix-core kernel takes the problem and fills use_mfma, mfma_ps and
 // the mfma_* fields (everything the launch needs, so that a forward call computes nothing).
 void mfma_plan(Geometry &g);
