@@ -121,6 +121,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-cold", action="store_true",
                     help="skip the leg that rotates through more buffers than the cache holds")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="profiling aid: every step of the run, warm-up included, rotates "
+                         "through the buffer pairs, so that a kernel trace of the run holds "
+                         "cold launches only")
     ap.add_argument("--no-host", action="store_true",
                     help="skip the three forward passes through host buffers")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -184,6 +188,20 @@ def main():
         assert len(tb) == args.steps and len(tc) == args.steps, (len(tb), len(tc))
         return wall_ms, sum(tb) / len(tb), sum(tc) / len(tc), sorted(tb), sorted(tc)
 
+    pair_bytes = xt.numel() * 4 + yt.numel() * 4
+    nsets = max(3, -(-4 * INFINITY_CACHE_BYTES // pair_bytes))
+    if args.cold_only:
+        sets = [(xt, yt)] + [(xt.clone(), torch.empty_like(yt)) for _ in range(nsets - 1)]
+        torch.cuda.synchronize()
+        for i in range(max(args.warmup, nsets)):
+            step(*sets[i % nsets])
+        cold_ms, cbin_ms, cconv_ms, _, _ = timed_steps(sets)
+        print(json.dumps({"cold_only": True, "workload": args.workload, "ms_per_step": cold_ms,
+                          "buffer_pairs": nsets, "kernel_us": {"binarize": cbin_ms * 1e3,
+                                                               "convolution": cconv_ms * 1e3}}))
+        conv.close()
+        return
+
     torch.cuda.synchronize()  # inputs were written on the default stream
     for _ in range(args.warmup):
         step()
@@ -220,8 +238,6 @@ def main():
     # the time it comes round again: the pairs together hold at least four times the cache.
     cold = None
     if not args.no_cold:
-        pair_bytes = xt.numel() * 4 + yt.numel() * 4
-        nsets = max(3, -(-4 * INFINITY_CACHE_BYTES // pair_bytes))
         sets = [(xt, yt)] + [(xt.clone(), torch.empty_like(yt)) for _ in range(nsets - 1)]
         torch.cuda.synchronize()
         for i in range(max(args.warmup, nsets)):
