@@ -243,8 +243,20 @@ def main():
         for i in range(max(args.warmup, nsets)):
             step(*sets[i % nsets])
         cold_ms, cbin_ms, cconv_ms, _, _ = timed_steps(sets)
+        # the binarize kernel alone over the same rotation: its input comes from HBM as in the
+        # cold steps, but no convolution output is waiting in the caches to be written back
+        # while it runs
+        for i in range(nsets):
+            conv.stage("binarize_data", src=sets[i][0], dst=sets[i][1])
+        conv.time_kernels(args.steps)
+        for i in range(args.steps):
+            conv.stage("binarize_data", src=sets[i % nsets][0], dst=sets[i % nsets][1])
+        torch.cuda.synchronize()
+        alone = conv.kernel_times(capi.OP_BINARIZE_DATA)
+        conv.time_kernels(0)
         cold = {"ms_per_step": cold_ms, "buffer_pairs": nsets, "bytes_per_pair": pair_bytes,
-                "kernel_us": {"binarize": cbin_ms * 1e3, "convolution": cconv_ms * 1e3},
+                "kernel_us": {"binarize": cbin_ms * 1e3, "convolution": cconv_ms * 1e3,
+                              "binarize_without_convolutions": 1e3 * sum(alone) / len(alone)},
                 "value": wf["nominal_ops"] / (cold_ms * 1e-3) / 1e9}
         del sets
 

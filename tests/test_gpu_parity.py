@@ -704,3 +704,21 @@ def test_random_problems_until_the_time_is_up(oracle):
         assert ok, "case %d %s formats %s (%s)" % (n, d, fmts, name)
         n += 1
     assert n >= 5
+
+
+@pytest.mark.parametrize("fmts", [NCHW, (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC)],
+                         ids=["nchw", "nhwc_out"])
+def test_streaming_output_stores(oracle, gpu, monkeypatch, fmts):
+    """The matrix-core kernel stores large outputs with the streaming cache policy (chosen
+    from the footprint at init; the full-size ResNet workload above takes it).  Forced on
+    here for small and ragged shapes: same bits, whatever the policy."""
+    monkeypatch.setenv("XNOR_NN_HIP_STREAM_DST", "1")
+    for name, mb in (("alexnet_conv4_mb256", 5), ("resnet_3x3_mb64", 1), ("vgg_512_mb32", 1)):
+        d, x, w = synth.make_workload(name, mb)
+        run_and_compare(oracle, d, x, w, fmts, device_tensors=True, gpu=gpu)
+    d = shapes.as_dims((2, 70, 100, 9, 7, 3, 3, 1, 1, 1, 1))  # ragged filters and planes
+    x = synth.normal(141, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    w = synth.normal(142, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    run_and_compare(oracle, d, x, w, fmts)

@@ -32,15 +32,15 @@ def hipcc():
     return exe
 
 
-def build(verbose=True, extra=()):
+def build(verbose=True, extra=(), out=OUT):
     sources = sorted(glob.glob(os.path.join(SRC, "*.hip")))
-    os.makedirs(os.path.dirname(OUT), exist_ok=True)
+    os.makedirs(os.path.dirname(out), exist_ok=True)
     cmd = [hipcc()] + FLAGS + list(extra) + [
-        "-I" + os.path.join(ROOT, "include"), "-I" + SRC] + sources + ["-o", OUT]
+        "-I" + os.path.join(ROOT, "include"), "-I" + SRC] + sources + ["-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    return OUT
+    return out
 
 
 if __name__ == "__main__":

@@ -91,7 +91,8 @@ def bind(lib, symbols):
 def library_path():
     """In-tree location of the HIP library built by ``xnor_nn_amd.build``."""
     here = os.path.dirname(os.path.abspath(__file__))
-    return os.path.join(here, "lib", "libxnor_nn.so")
+    # XNOR_NN_AMD_LIBRARY names another build of the same library (measurements of variants)
+    return os.environ.get("XNOR_NN_AMD_LIBRARY") or os.path.join(here, "lib", "libxnor_nn.so")
 
 
 _LIB = None

@@ -52,6 +52,14 @@ constexpr int LDS_LIMIT = 160 * 1024;    // a gfx950 workgroup may take the whol
 constexpr int LDS_DEFAULT = 64 * 1024;   // above this the kernel has to ask for it
 constexpr int LDS_TWO_PER_CU = 80 * 1024;
 constexpr int MAX_DEVICES = 64;
+// Cache policy of the output stores: 0 = write-back through L2 and the Infinity Cache, 2 = the
+// "nt" bit, streaming.  Streaming stores keep an output that will not be read soon from
+// pushing the next input out of the 256 MB Infinity Cache (and from sitting there as dirty
+// lines that the next kernel's reads have to wait for): ResNet 3x3 56x56 MB 64, 205 MB in and
+// 205 MB out, 130 -> 105 us per forward pass (the binarize kernel of the next pass 56 -> 31 us,
+// this kernel 64.5 -> 66.4 us).  Where input and output fit the cache together, write-back is
+// faster (AlexNet conv4 MB 256: this kernel 23.6 us against 28.8 us streaming).
+constexpr int STORE_WRITE_BACK = 0, STORE_STREAMING = 2;
 
 // First and last input pixel (flattened index) that the tile of mt output pixels starting
 // at tile*mt can touch with an in-bounds tap: from the start of the first input row of its
@@ -643,8 +651,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // 16-byte stores need filter runs that start on a 16-byte boundary
     const bool vec4_ok = !nchw && (g.oc & 3) == 0
         && ((size_t)(RAW ? static_cast<void *>(popc) : static_cast<void *>(dst)) & 15) == 0;
-    auto store_tile = [&](auto check_filters, auto planar) {
+    auto store_tile = [&](auto check_filters, auto planar, auto policy) {
         constexpr bool CHECK = decltype(check_filters)::value, NCHW = decltype(planar)::value;
+        constexpr int STORE_AUX = decltype(policy)::value;
 #pragma unroll
         for (int os = 0; os < 2; os++) {
 #pragma unroll
@@ -673,16 +682,16 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                                     v[2 * q + 1], false, false);
                             // r[0]: filter f, pixels 64q + lane; r[1]: filter f + 4
                             if (!CHECK || f < g.oc)
-                                __builtin_amdgcn_raw_buffer_store_b32(r[0], outbuf, off2[q], soff, 0);
+                                __builtin_amdgcn_raw_buffer_store_b32(r[0], outbuf, off2[q], soff, STORE_AUX);
                             if (!CHECK || f + 4 < g.oc)
                                 __builtin_amdgcn_raw_buffer_store_b32(r[1], outbuf, off2[q],
-                                        soff + 4u * fstep, 0);
+                                        soff + 4u * fstep, STORE_AUX);
                         }
                     }
 #pragma unroll
                     for (int ps = NCHW ? (PS / 2) * 2 : 0; ps < PS; ps++) {
                         const uint32_t voff = CHECK && f + lane_hi * 4 >= g.oc ? DROP : off1[ps];
-                        __builtin_amdgcn_raw_buffer_store_b32(v[ps], outbuf, voff, soff, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32(v[ps], outbuf, voff, soff, STORE_AUX);
                     }
                 }
             }
@@ -694,7 +703,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     // 128 contiguous bytes of 8 pixels instead of 32 bytes of 32 pixels.  Rows of 144 bytes
     // keep both sides free of bank conflicts.  A piece past OC (OC is a multiple of 4 here)
     // or a pixel past the end gets an offset outside the buffer.
-    auto store_lines_nhwc = [&]() {
+    auto store_lines_nhwc = [&](auto policy) {
+        constexpr int STORE_AUX = decltype(policy)::value;
         float *mine = turn_lds + wave * (32 * TURN_ROW);
         const int piece = lane & 7, prow = lane >> 3;
         const uint32_t left = g.npix_out - p_first; // pixels of the tile that exist
@@ -724,7 +734,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
                     const uint32_t in_tile = (uint32_t)(ps * 32 + 8 * j); // + prow
                     const uint32_t voff = in_tile + (uint32_t)prow < left ? base : DROP;
                     __builtin_amdgcn_raw_buffer_store_b128(r, outbuf, voff,
-                            in_tile * (uint32_t)g.oc * 4u, 0);
+                            in_tile * (uint32_t)g.oc * 4u, STORE_AUX);
                 }
             }
         }
@@ -732,16 +742,24 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const bool all_filters = chunk * NT + (wave + 1) * 64 <= g.oc; // wave-uniform
     if constexpr (!RAW) {
         if (vec4_ok) {
-            store_lines_nhwc();
+            if (g.stream_dst) store_lines_nhwc(std::integral_constant<int, STORE_STREAMING>{});
+            else store_lines_nhwc(std::integral_constant<int, STORE_WRITE_BACK>{});
             return;
         }
     }
+    using WriteBack = std::integral_constant<int, STORE_WRITE_BACK>;
+    using Streaming = std::integral_constant<int, STORE_STREAMING>;
     if (nchw) {
-        if (all_filters) store_tile(std::false_type{}, std::true_type{});
-        else store_tile(std::true_type{}, std::true_type{});
+        if (g.stream_dst) {
+            if (all_filters) store_tile(std::false_type{}, std::true_type{}, Streaming{});
+            else store_tile(std::true_type{}, std::true_type{}, Streaming{});
+        } else {
+            if (all_filters) store_tile(std::false_type{}, std::true_type{}, WriteBack{});
+            else store_tile(std::true_type{}, std::true_type{}, WriteBack{});
+        }
     } else {
-        if (all_filters) store_tile(std::false_type{}, std::false_type{});
-        else store_tile(std::true_type{}, std::false_type{});
+        if (all_filters) store_tile(std::false_type{}, std::false_type{}, WriteBack{});
+        else store_tile(std::true_type{}, std::false_type{}, WriteBack{});
     }
 }
 
@@ -1016,9 +1034,21 @@ void mfma_plan(Geometry &g) {
     g.mfma_ps = mfma_tile_blocks(g);
     g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
     g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
+    g.stream_dst = 0;
     g.mfma_parts = 1;
     g.mfma_lds = g.mfma_wbytes = 0;
     if (!g.use_mfma) return;
+    // Output stores stream past the caches when the input of the next forward pass and this
+    // output cannot both stay in the 256 MB Infinity Cache, and the runs of one filter start
+    // on 64-byte boundaries: with ragged planes (13 x 13, 27 x 27) streaming stores leave
+    // partial lines behind and cost the kernel 15 to 25 %, more than the next pass gains.
+    // XNOR_NN_HIP_STREAM_DST=0|1 overrides, for measurements.
+    const uint64_t in_bytes = (uint64_t)g.npix_in * g.ic * 4u;
+    const uint64_t out_bytes = (uint64_t)g.npix_out * g.oc * 4u;
+    const uint32_t run_bytes = g.dst_fmt == xnor_nn_data_format_nchw ? (uint32_t)g.ohw * 4u
+                                                                     : (uint32_t)g.oc * 4u;
+    g.stream_dst = in_bytes + out_bytes > (200ull << 20) && run_bytes % 64 == 0 ? 1 : 0;
+    if (const char *e = getenv("XNOR_NN_HIP_STREAM_DST")) g.stream_dst = e[0] == '1' ? 1 : 0;
     g.mfma_steps = steps_per_tap(g);
     g.mfma_pair = pair_taps(g) ? 1 : 0;
     g.mfma_parts = channel_parts(g);

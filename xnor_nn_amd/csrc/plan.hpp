@@ -68,6 +68,7 @@ struct Geometry {
     // per pair of taps), tap pairing, channel parts, input pixels a tile stages at most, LDS
     // bytes per workgroup, bytes of the weight fragments
     int mfma_steps, mfma_pair, mfma_parts, mfma_rows;
+    int stream_dst;             // 1: the matrix-core kernel stores its output with the nt bit
     uint32_t mfma_lds, mfma_wbytes;
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
