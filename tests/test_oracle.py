@@ -1,6 +1,8 @@
 """Pins the CPU oracle (oracle/xnor_oracle.c) without needing the upstream library:
 the upstream tests' known-answer vectors, closed forms, brute force on small inputs, and
 the committed digests of the upstream library's outputs (tests/golden/golden.json)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -220,3 +222,20 @@ def test_binarize_weights_float_closed_forms(oracle):
     assert np.array_equal(oracle.binarize_weights_float(s, w).view(np.uint32),
                           want.view(np.uint32))
     assert abs(float(mean) - float(np.mean(w.astype(np.float64)))) < 1e-7
+
+
+def test_oracle_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """tests/oracle_sanitize.c compiles the oracle's source into a host program with
+    -fsanitize=address,undefined and runs every stage over small and ragged shapes in all
+    eight layout combinations on exactly sized heap buffers: an index outside a tensor or
+    undefined arithmetic in the restatement ends it with a report."""
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = tmp_path / "oracle_sanitize"
+    subprocess.check_call(["gcc", "-std=c11", "-O1", "-g", "-fopenmp", "-ffp-contract=off",
+                           "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                           "-static-libasan", os.path.join(here, "oracle_sanitize.c"), "-lm",
+                           "-o", str(exe)])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, (out.stdout[-1000:], out.stderr[-3000:])
+    assert out.stdout.strip().endswith("0 bad")
