@@ -722,3 +722,27 @@ def test_streaming_output_stores(oracle, gpu, monkeypatch, fmts):
     w = synth.normal(142, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
         d["oc"], d["ic"], d["kh"], d["kw"])
     run_and_compare(oracle, d, x, w, fmts)
+
+
+@pytest.mark.parametrize("t,fmts", [
+    ((40, 384, 256, 13, 13, 3, 3, 1, 1, 1, 1), NCHW),                    # conv4: 212 blocks, 27 per XCD
+    ((7, 384, 256, 13, 13, 3, 3, 1, 1, 1, 1), NCHW),                     # fewer blocks than XCDs x 4
+    ((3, 96, 130, 27, 27, 5, 5, 1, 1, 2, 2), NCHW),                      # paired taps, ragged filters
+    ((5, 64, 64, 28, 28, 3, 3, 2, 2, 1, 1), (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC)),
+    ((2, 512, 200, 14, 14, 3, 3, 1, 1, 1, 1), NCHW),                     # 8 steps per tap
+    ((1, 33, 32, 5, 5, 3, 3, 1, 1, 1, 1), NCHW),                         # a single pixel block
+], ids=lambda v: shapes.shape_id(v) if len(v) == 11 else "fmt%d%d%d" % v)
+def test_two_tile_sizes_in_one_launch(oracle, monkeypatch, t, fmts):
+    """The matrix-core kernel with four-block tiles for the first workgroups of an XCD and
+    two-block tiles for the rest (chosen by size at init; the full-size conv4 workload above
+    takes it), forced on for problems whose XCD ranges end raggedly or hold no big tile."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_MIX", "1")
+    d = shapes.as_dims(t)
+    x = synth.normal(151, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::6] = 0.0
+    w = synth.normal(152, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    name = make(d, w, fmts).kernel_name(0)
+    assert "PS=4+2" in name, name
+    run_and_compare(oracle, d, x, w, fmts)

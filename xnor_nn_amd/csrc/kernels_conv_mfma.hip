@@ -61,16 +61,13 @@ constexpr int MAX_DEVICES = 64;
 // faster (AlexNet conv4 MB 256: this kernel 23.6 us against 28.8 us streaming).
 constexpr int STORE_WRITE_BACK = 0, STORE_STREAMING = 2;
 
-// First and last input pixel (flattened index) that the tile of mt output pixels starting
-// at tile*mt can touch with an in-bounds tap: from the start of the first input row of its
-// first pixel to the end of the last input row of its last pixel (with a stride above 1
+// First and last input pixel (flattened index) that a tile of the output pixels
+// [p_first, p_end) can touch with an in-bounds tap: from the start of the first input row of
+// its first pixel to the end of the last input row of its last pixel (with a stride above 1
 // the span also holds the input pixels the stride skips).
-__host__ __device__ inline void tile_span(const Geometry &g, uint32_t tile, uint32_t mt,
+__host__ __device__ inline void tile_span(const Geometry &g, uint32_t p_first, uint32_t p_end,
         int &lo, int &hi) {
-    const uint32_t p_first = tile * mt;
-    uint32_t p_last = p_first + mt;
-    if (p_last > g.npix_out) p_last = g.npix_out;
-    p_last -= 1;
+    const uint32_t p_last = p_end - 1;
     const uint32_t i0 = g.div_ohw.div(p_first), i1 = g.div_ohw.div(p_last);
     const int oh0 = (int)g.div_ow.div(p_first - i0 * g.ohw);
     const int oh1 = (int)g.div_ow.div(p_last - i1 * g.ohw);
@@ -193,15 +190,17 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
 // DEEP (more than 1024 channels): the channels of a pixel are cut into ic_parts parts of
 // 64*KS, and every (tap, part) is walked like a tap of its own whose rows start
 // 32*KS bytes further into the same LDS rows.
+// One tile: the output pixels [p_first, min(p_first + 32*PS, p_limit)) x the 256 filters of
+// filter chunk `chunk`.
 template <int KS, int PS, bool RAW, bool PAIR, bool DEEP>
-__global__ __launch_bounds__(256, 2)
-void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
+__device__ __forceinline__
+void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
         float *__restrict__ dst, int32_t *__restrict__ popc,
-        const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
-        const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
-        float *__restrict__ k_out, const float inv_khw, const int ic_parts,
-        const uint32_t wfrag_bytes) {
+        const Geometry &g, const int max_rows, const FastDiv &div_xw,
+        const float *__restrict__ a_plane, float *__restrict__ k_out, const float inv_khw,
+        const int ic_parts, const uint32_t wfrag_bytes, const uint32_t p_first,
+        const uint32_t p_limit, const int chunk) {
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
@@ -231,20 +230,12 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroups are dealt to the eight XCDs round-robin: unit (b % 8) * units_per_xcd + b / 8
-    // gives each XCD one contiguous range of tiles, so the input rows two neighbouring tiles
-    // share and the output cache lines they both write into meet in one L2.
-    const uint32_t unit = (blockIdx.x & 7) * units_per_xcd + (blockIdx.x >> 3);
-    if (unit >= units) return;
-    const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
-    const int chunk = unit - tile * oc_chunks;
     // "taps" below are the units the main loop walks over: kernel taps, or pairs of them
     const int taps = PAIR ? (g.kh * g.kw + 1) / 2 : DEEP ? g.kh * g.kw * ic_parts : g.kh * g.kw;
 
     // ---- which input pixels does the tile touch ------------------------------------------
-    const uint32_t p_first = tile * MT;
     int lo, hi;
-    tile_span(g, tile, MT, lo, hi);
+    tile_span(g, p_first, min(p_first + (uint32_t)MT, p_limit), lo, hi);
     const int nrows = min(hi - lo + 1, max_rows);
 
     // ---- the 32*PS output pixels of the tile, one per lane and 32-pixel block -----------------
@@ -257,8 +248,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 #pragma unroll
     for (int ps = 0; ps < PS; ps++) {
         pix[ps] = p_first + ps * 32 + (lane & 31);
-        live[ps] = pix[ps] < g.npix_out;
-        const uint32_t pc = live[ps] ? pix[ps] : g.npix_out - 1;
+        live[ps] = pix[ps] < p_limit;
+        const uint32_t pc = live[ps] ? pix[ps] : p_limit - 1;
         img[ps] = g.div_ohw.div(pc);
         rem[ps] = pc - img[ps] * g.ohw;
         const int oh = (int)g.div_ow.div(rem[ps]);
@@ -643,9 +634,9 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
 #pragma unroll
     for (int q = 0; q < PS / 2; q++) {
         const uint32_t p64 = p_first + q * 64 + lane;
-        const uint32_t pc = p64 < g.npix_out ? p64 : g.npix_out - 1;
+        const uint32_t pc = p64 < p_limit ? p64 : p_limit - 1;
         const uint32_t im = g.div_ohw.div(pc);
-        off2[q] = p64 < g.npix_out
+        off2[q] = p64 < p_limit
             ? (im * (uint32_t)g.oc * (uint32_t)g.ohw + (pc - im * g.ohw)) * 4u : DROP;
     }
     // 16-byte stores need filter runs that start on a 16-byte boundary
@@ -707,7 +698,7 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         constexpr int STORE_AUX = decltype(policy)::value;
         float *mine = turn_lds + wave * (32 * TURN_ROW);
         const int piece = lane & 7, prow = lane >> 3;
-        const uint32_t left = g.npix_out - p_first; // pixels of the tile that exist
+        const uint32_t left = p_limit - p_first; // pixels of the tile that exist
 #pragma unroll
         for (int os = 0; os < 2; os++) {
             const uint32_t fpiece = (uint32_t)(chunk * NT + (wave * 2 + os) * 32 + 4 * piece);
@@ -760,6 +751,56 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     } else {
         if (all_filters) store_tile(std::false_type{}, std::false_type{}, WriteBack{});
         else store_tile(std::true_type{}, std::false_type{}, WriteBack{});
+    }
+}
+
+// Which tile a workgroup takes.  Workgroups are dealt to the eight XCDs round-robin, so
+// workgroup b runs on XCD b % 8 and is the (b / 8)-th of that XCD.
+//
+// PSB == 0, one tile size: unit (b % 8) * units_per_xcd + b / 8 gives each XCD one contiguous
+// range of tiles, so the input rows two neighbouring tiles share and the output cache lines
+// they both write into meet in one L2.  A unit is a (tile, filter chunk) pair.
+//
+// PSB > 0, two tile sizes (one filter chunk only): XCD x owns the pixel blocks
+// [x * blocks_per_xcd, (x+1) * blocks_per_xcd); its first big_per_xcd workgroups take PS
+// blocks each, the following ones PSB blocks each.  The hardware starts workgroups in the
+// order of their index and the matrix pipe serves the older wave of a SIMD first, so on a
+// compute unit that holds two workgroups the one with the small tile is the one that
+// finishes last: its epilogue, the only one nothing overlaps, is the short one.
+template <int KS, int PS, int PSB, bool RAW, bool PAIR, bool DEEP>
+__global__ __launch_bounds__(256, 2)
+void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
+        const float *__restrict__ alpha, const float *__restrict__ kplane,
+        float *__restrict__ dst, int32_t *__restrict__ popc,
+        const Geometry g, const int max_rows, const int oc_chunks, const uint32_t units,
+        const uint32_t units_per_xcd, const FastDiv div_xw, const float *__restrict__ a_plane,
+        float *__restrict__ k_out, const float inv_khw, const int ic_parts,
+        const uint32_t wfrag_bytes, const uint32_t big_per_xcd, const uint32_t blocks_per_xcd) {
+    const uint32_t xcd = blockIdx.x & 7, nth = blockIdx.x >> 3;
+    if constexpr (PSB == 0) {
+        const uint32_t unit = xcd * units_per_xcd + nth;
+        if (unit >= units) return;
+        const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
+        const int chunk = unit - tile * oc_chunks;
+        conv_tile<KS, PS, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g, max_rows,
+                div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, tile * (32u * PS),
+                g.npix_out, chunk);
+    } else {
+        const uint32_t first = xcd * blocks_per_xcd; // pixel blocks of this XCD: [first, last)
+        const uint32_t p_limit = min((first + blocks_per_xcd) * 32u, g.npix_out);
+        if (nth < big_per_xcd) {
+            const uint32_t p_first = (first + nth * PS) * 32u;
+            if (p_first >= p_limit) return;
+            conv_tile<KS, PS, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g,
+                    max_rows, div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, p_first,
+                    p_limit, 0);
+        } else {
+            const uint32_t p_first = (first + big_per_xcd * PS + (nth - big_per_xcd) * PSB) * 32u;
+            if (p_first >= p_limit) return;
+            conv_tile<KS, PSB, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g,
+                    max_rows, div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, p_first,
+                    p_limit, 0);
+        }
     }
 }
 
@@ -852,26 +893,27 @@ int steps_per_tap(const Geometry &g) {
 }
 int oc_subblocks(const Geometry &g) { return ((g.oc + NT - 1) / NT) * (NT / 32); }
 
-// Largest number of input pixels any tile of mt output pixels touches.  The offset of a
-// tile within its image repeats after at most OHW tiles, so that many (plus the last,
-// possibly short, tile) are enough to look at.
-int max_tile_rows(const Geometry &g, uint32_t mt) {
-    const uint32_t tiles = (g.npix_out + mt - 1) / mt;
-    const uint32_t look = tiles < (uint32_t)g.ohw + 1 ? tiles : (uint32_t)g.ohw + 1;
+// Largest number of input pixels any tile of mt output pixels touches.  Tiles start at
+// multiples of `step` pixels (their own size for a launch with one tile size, 32 for a launch
+// with two); the offset of a tile within its image repeats after at most OHW starts, so that
+// many (plus the last, possibly short, tile) are enough to look at.
+int max_tile_rows(const Geometry &g, uint32_t mt, uint32_t step = 0) {
+    if (step == 0) step = mt;
+    const uint32_t starts = (g.npix_out + step - 1) / step;
+    const uint32_t look = starts < (uint32_t)g.ohw + 1 ? starts : (uint32_t)g.ohw + 1;
     int most = 1;
-    for (uint32_t t = 0; t < look; t++) {
+    auto see = [&](uint32_t t) {
         int lo, hi;
-        tile_span(g, t, mt, lo, hi);
+        const uint32_t first = t * step;
+        tile_span(g, first, first + mt < g.npix_out ? first + mt : g.npix_out, lo, hi);
         if (hi - lo + 1 > most) most = hi - lo + 1;
-    }
-    int lo, hi;
-    tile_span(g, tiles - 1, mt, lo, hi);
-    if (hi - lo + 1 > most) most = hi - lo + 1;
+    };
+    for (uint32_t t = 0; t < look; t++) see(t);
+    see(starts - 1);
     return most;
 }
 
-size_t lds_bytes(const Geometry &g, int ps) {
-    const size_t rows = (size_t)max_tile_rows(g, 32 * ps);
+size_t lds_bytes_for(const Geometry &g, size_t rows, int ps) {
     const size_t row_bytes = pair_taps(g) ? g.xw * 16
         : channel_parts(g) * steps_per_tap(g) * 32 + ROW_PAD;
     size_t bytes = TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
@@ -879,6 +921,9 @@ size_t lds_bytes(const Geometry &g, int ps) {
     if (g.dst_fmt == xnor_nn_data_format_nhwc && (g.oc & 3) == 0) // turn-around rows, 4 waves
         bytes = ((bytes + 15) & ~(size_t)15) + 4 * 32 * TURN_ROW * sizeof(float);
     return bytes;
+}
+size_t lds_bytes(const Geometry &g, int ps) {
+    return lds_bytes_for(g, (size_t)max_tile_rows(g, 32 * ps), ps);
 }
 
 // 32-pixel blocks per tile, by a model of the kernel's time in core cycles that was fitted to
@@ -936,13 +981,21 @@ int pick_ps(const Geometry &g) {
     return best;
 }
 
-template <int KS, int PS, bool PAIR, bool DEEP = false>
+template <int KS, int PS, bool PAIR, bool DEEP = false, int PSB = 0>
 hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     const int chunks = (g.oc + NT - 1) / NT;
     const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
-    const uint32_t units = tiles * chunks, per_xcd = (units + 7) / 8;
+    const uint32_t units = tiles * chunks;
+    uint32_t per_xcd = (units + 7) / 8; // workgroups per XCD
+    uint32_t big = 0, blocks = 0;
+    if constexpr (PSB > 0) { // two tile sizes: see the kernel
+        blocks = g.mfma_blocks_per_xcd;
+        big = g.mfma_big_per_xcd;
+        const uint32_t rest = blocks > big * PS ? blocks - big * PS : 0;
+        per_xcd = big + (rest + PSB - 1) / PSB;
+    }
     const dim3 grid(per_xcd * 8), block(256);
     const int rows = g.mfma_rows;
     const size_t lds = g.mfma_lds;
@@ -957,8 +1010,8 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         std::atomic<size_t> &have = granted[popc ? 1 : 0][dev];
         if (lds > have.load(std::memory_order_acquire)) {
             const void *fn = popc
-                ? (const void *)conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>
-                : (const void *)conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>;
+                ? (const void *)conv_mfma_fp4_kernel<KS, PS, PSB, true, PAIR, DEEP>
+                : (const void *)conv_mfma_fp4_kernel<KS, PS, PSB, false, PAIR, DEEP>;
             const hipError_t e = hipFuncSetAttribute(fn,
                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return e;
@@ -966,15 +1019,15 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         }
     }
     if (popc)
-        launch_kernel(conv_mfma_fp4_kernel<KS, PS, true, PAIR, DEEP>, grid, block, lds, s, ev,
-                xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
+        launch_kernel(conv_mfma_fp4_kernel<KS, PS, PSB, true, PAIR, DEEP>, grid, block, lds, s,
+                ev, xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
-                g.mfma_wbytes);
+                g.mfma_wbytes, big, blocks);
     else
-        launch_kernel(conv_mfma_fp4_kernel<KS, PS, false, PAIR, DEEP>, grid, block, lds, s, ev,
-                xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
+        launch_kernel(conv_mfma_fp4_kernel<KS, PS, PSB, false, PAIR, DEEP>, grid, block, lds, s,
+                ev, xbits, wf, alpha, k, dst, popc, g, rows, chunks, units, per_xcd,
                 FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, parts,
-                g.mfma_wbytes);
+                g.mfma_wbytes, big, blocks);
     return hipGetLastError();
 }
 
@@ -994,6 +1047,12 @@ template <int KS, bool PAIR = false>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
+    if (g.mfma_ps_small > 0) { // four blocks for the first workgroup of a CU, two for the second
+        if constexpr (KS < 16 && !(PAIR && KS >= 5))
+            return launch_mfma<KS, 4, PAIR, false, 2>(g, xbits, wfrag, alpha, k, dst, popc,
+                    a_or_null, k_out, s, ev);
+        return hipErrorInvalidValue;
+    }
     switch (g.mfma_ps) {
     case 1: return launch_mfma<KS, 1, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
     case 2: return launch_mfma<KS, 2, PAIR>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);
@@ -1034,6 +1093,8 @@ void mfma_plan(Geometry &g) {
     g.mfma_ps = mfma_tile_blocks(g);
     g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
     g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
+    g.mfma_ps_small = 0;
+    g.mfma_big_per_xcd = g.mfma_blocks_per_xcd = 0;
     g.stream_dst = 0;
     g.mfma_parts = 1;
     g.mfma_lds = g.mfma_wbytes = 0;
@@ -1055,6 +1116,31 @@ void mfma_plan(Geometry &g) {
     g.mfma_rows = max_tile_rows(g, 32 * g.mfma_ps);
     g.mfma_lds = (uint32_t)lds_bytes(g, g.mfma_ps);
     g.mfma_wbytes = (uint32_t)mfma_weight_bytes(g);
+    // Two tile sizes in one launch (see the kernel): worth it when every compute unit gets
+    // more than four and at most six pixel blocks, i.e. when equal tiles would give it two
+    // workgroups of three that finish together.  Needs one filter chunk, the four-block
+    // variant, and room for two workgroups in a CU's LDS.  XNOR_NN_HIP_MFMA_MIX=0|1 overrides
+    // the size rule (for measurements), a forced tile size switches it off.
+    const uint32_t blocks = (g.npix_out + 31) / 32, blocks_per_xcd = (blocks + 7) / 8;
+    const uint32_t cus_per_xcd = (uint32_t)(g.cus + 7) / 8;
+    bool mix = blocks_per_xcd > 4 * cus_per_xcd && blocks_per_xcd <= 6 * cus_per_xcd;
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_MIX")) mix = e[0] == '1';
+    if (getenv("XNOR_NN_HIP_MFMA_PS") || g.oc > NT || g.mfma_parts > 1 || g.mfma_steps >= 16
+            || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4))
+        mix = false;
+    if (mix) {
+        const int rows = max_tile_rows(g, 32 * 4, 32);
+        const size_t lds = lds_bytes_for(g, (size_t)rows, 4);
+        if (lds <= (size_t)LDS_TWO_PER_CU) {
+            g.mfma_ps = 4;
+            g.mfma_ps_small = 2;
+            g.mfma_blocks_per_xcd = blocks_per_xcd;
+            const uint32_t fit = blocks_per_xcd / 4; // whole four-block tiles in an XCD's range
+            g.mfma_big_per_xcd = fit < cus_per_xcd ? fit : cus_per_xcd;
+            g.mfma_rows = rows;
+            g.mfma_lds = (uint32_t)lds;
+        }
+    }
 }
 
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,
@@ -1070,6 +1156,9 @@ const char *mfma_kernel_name(const Geometry &g) {
     if (g.mfma_parts > 1)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d,PARTS=%d>",
                 g.mfma_steps, g.mfma_ps, g.mfma_parts);
+    else if (g.mfma_ps_small > 0)
+        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d+%d%s>", g.mfma_steps,
+                g.mfma_ps, g.mfma_ps_small, g.mfma_pair ? ",PAIR" : "");
     else
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", g.mfma_steps,
                 g.mfma_ps, g.mfma_pair ? ",PAIR" : "");

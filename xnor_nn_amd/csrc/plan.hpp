@@ -63,6 +63,10 @@ struct Geometry {
     int cus;                    // compute units of the device (256 if it cannot be asked)
     int use_mfma;               // 1: stage 3 runs the FP4 matrix-core kernel
     int mfma_ps;                // its tile size in 32-pixel blocks (1..4)
+    int mfma_ps_small;          // > 0: a launch with two tile sizes; the later workgroups of an
+                                // XCD take this many blocks (see the kernel)
+    uint32_t mfma_big_per_xcd;  // ... after this many workgroups with mfma_ps blocks,
+    uint32_t mfma_blocks_per_xcd; // out of this many pixel blocks per XCD
     size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
     // the matrix-core kernel's variant and sizes, fixed once by mfma_plan: steps per tap (or
     // per pair of taps), tap pairing, channel parts, input pixels a tile stages at most, LDS
