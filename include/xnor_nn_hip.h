@@ -119,7 +119,8 @@ xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz);
  * descriptor's stream and returns (no allocation, no free, no memset, no synchronisation),
  * and writes the same bits as xnor_nn_binarize_weights_float.  The 256 partial sums live in
  * a 1 KB device array that is part of the library and stays on every GPU the library has
- * run on until the process ends.  Every call on a GPU shares that array: calls that overlap
+ * run on until the process ends (its device address is looked up once per GPU, by
+ * xnor_nn_init_convolution or by the first call here, whichever comes first).  Every call on a GPU shares that array: calls that overlap
  * on one GPU (two streams, two threads) race on it and must be ordered by the caller.
  * More than XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS weights, or a host pointer that is null, is
  * refused with xnor_nn_error_invalid_input and a line on stderr. */

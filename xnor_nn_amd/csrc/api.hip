@@ -457,10 +457,16 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
     {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n,
-                    hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+                    hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) {
             g.cus = n;
-        else
+            // the device address of the library's static partial-sum array is looked up here,
+            // once per device, so that xnor_nn_hip_binarize_weights_float_noalloc itself
+            // only reads it back (it may be called where nothing may be set up any more)
+            float *unused = nullptr;
+            if (weights_float_scratch(&unused) != hipSuccess) (void)hipGetLastError();
+        } else {
             (void)hipGetLastError();
+        }
     }
     mfma_plan(g);
     g.wfrag_offset = (bit_bytes + 255) / 256 * 256;
