@@ -654,12 +654,13 @@ def test_linearity_of_scaling_at_full_size(gpu):
     conv.close()
 
 
-def test_random_problems_until_the_time_is_up(oracle):
+def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
     """Fifteen seconds of seeded random problems larger than the ones above (channel counts
     around the 32/64/1024 boundaries up to 2048, kernels 1..9, strides 1..4, paddings 0..4,
-    images up to 43 x 43, every layout combination, inputs with exact zeros of both signs):
-    dst and the raw popcounts against the oracle, bit for bit, stopping at the first
-    mismatch."""
+    images up to 43 x 43, every layout combination, inputs with exact zeros of both signs;
+    every third problem with the two-tile-size launch forced on, every fourth with streaming
+    output stores): dst and the raw popcounts against the oracle, bit for bit, stopping at
+    the first mismatch."""
     import time
     rng = np.random.default_rng(20251)
     t_end = time.time() + 15.0
@@ -693,7 +694,15 @@ def test_random_problems_until_the_time_is_up(oracle):
         xs = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if fmts[0] == capi.FMT_NHWC else x
         ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
         want = oracle.forward(oracle_shape(oracle, d, fmts), xs, ws)
-        print("case", n, d, fmts, flush=True)
+        # launch options that the library otherwise picks by problem size
+        forced = {"XNOR_NN_HIP_MFMA_MIX": "1" if n % 3 == 2 else None,
+                  "XNOR_NN_HIP_STREAM_DST": "1" if n % 4 == 3 else None}
+        for key, value in forced.items():
+            if value is None:
+                monkeypatch.delenv(key, raising=False)
+            else:
+                monkeypatch.setenv(key, value)
+        print("case", n, d, fmts, {k: v for k, v in forced.items() if v}, flush=True)
         conv = make(d, ws, fmts)
         dst = np.empty(want["dst"].shape, np.float32)
         conv.forward(xs, dst)
