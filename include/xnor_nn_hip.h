@@ -89,7 +89,7 @@ xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
         xnor_nn_resources_t res, int32_t *popc);
 
 /* Name of the kernel variant an executor of this descriptor launches (stage: one of
- * xnor_nn_operation_t), e.g. "conv_xnor_popc<XW=12,Q=16>"; the counterpart of the
+ * xnor_nn_operation_t), e.g. "conv_mfma_fp4_kernel<KS=6,PS=4+2>"; the counterpart of the
  * reference's XNOR_NN_VERBOSE line (reference src/utils/convolution_logger.hpp:99-152).
  * Returns the length written (without terminator). */
 int xnor_nn_hip_kernel_name(const xnor_nn_convolution_t *c, int stage,

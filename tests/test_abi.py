@@ -219,3 +219,56 @@ def test_stage_fusion_switch_and_table_bookkeeping_without_a_gpu():
     res = capi.Resources()
     lib.xnor_nn_free_resources(res)
     lib.xnor_nn_destroy_convolution(C.byref(c))
+
+
+def kernel_names(shape, fmts=(capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NCHW)):
+    """(binarize kernel, convolution kernel) the library plans for a shape
+    (mb, oc, ic, ih, iw, kh, kw, sh, sw, ph, pw); planning needs no GPU (256 CUs assumed)."""
+    lib = capi.load()
+    c = capi.ConvolutionDesc()
+    assert lib.xnor_nn_init_convolution(C.byref(c), capi.ALGORITHM_BCAST, *fmts, *shape) \
+        == capi.SUCCESS
+    buf = C.create_string_buffer(96)
+    out = []
+    for stage in (capi.OP_BINARIZE_DATA, capi.OP_CONVOLUTION_FORWARD):
+        lib.xnor_nn_hip_kernel_name(C.byref(c), stage, buf, len(buf))
+        out.append(buf.value.decode())
+    lib.xnor_nn_destroy_convolution(C.byref(c))
+    return tuple(out)
+
+
+def test_kernel_variants_planned_for_known_shapes(monkeypatch):
+    """The counterpart of the reference's dispatcher (reference src/bcast_convolution.hpp:13-38,
+    src/bcast_convolution.cpp:14-43: exact-match table of shapes -> unrolled kernel, else the
+    runtime-shape kernel): which kernel variant each of the five benchmark workloads and the
+    boundary shapes get, decided at init from the shape alone."""
+    for key in ("XNOR_NN_HIP_CONV", "XNOR_NN_HIP_MFMA_PS", "XNOR_NN_HIP_MFMA_MIX",
+                "XNOR_NN_HIP_MFMA_PAIR", "XNOR_NN_HIP_NHWC", "XNOR_NN_HIP_STREAM_DST"):
+        monkeypatch.delenv(key, raising=False)
+    conv4 = (256, 384, 13, 13, 3, 3, 1, 1, 1, 1)
+    assert kernel_names((1,) + conv4) == ("binarize_nchw_kernel", "conv_mfma_fp4_kernel<KS=6,PS=1>")
+    # 5.3 pixel blocks per compute unit: two tile sizes in one launch
+    assert kernel_names((256,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4+2>"
+    assert kernel_names((1024,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4>"
+    # 96 channels = three words: two taps share three steps
+    assert kernel_names((128, 256, 96, 27, 27, 5, 5, 1, 1, 2, 2))[1] \
+        == "conv_mfma_fp4_kernel<KS=3,PS=4,PAIR>"
+    assert kernel_names((64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
+        == "conv_mfma_fp4_kernel<KS=4,PS=4>"
+    assert kernel_names((32, 512, 512, 28, 28, 3, 3, 1, 1, 1, 1))[1] \
+        == "conv_mfma_fp4_kernel<KS=8,PS=4>"
+    # more than 1024 channels: channel parts; more than 4096: no matrix cores
+    assert re.fullmatch(r"conv_mfma_fp4_kernel<KS=1[26],PS=\d,PARTS=\d>",
+                        kernel_names((2, 64, 2048, 8, 8, 3, 3, 1, 1, 1, 1))[1])
+    deep = kernel_names((1, 32, 8200, 4, 4, 1, 1, 1, 1, 0, 0))
+    assert deep[0] == "binarize_generic_kernel" and deep[1] == "conv_xnor_popc_kernel<XW=0,Q=16>"  # XW=0: word count at run time
+    # kernels wider than 32 taps keep their tap masks in 32 bits: XNOR/popcount kernel
+    assert kernel_names((1, 16, 32, 40, 40, 33, 33, 1, 1, 0, 0))[1].startswith("conv_xnor_popc")
+    # input layouts
+    nhwc = (capi.FMT_NHWC, capi.FMT_OIHW, capi.FMT_NCHW)
+    assert kernel_names((4,) + conv4, nhwc)[0] == "binarize_nhwc_tiled_kernel"
+    assert kernel_names((1, 32, 2048, 6, 6, 3, 3, 1, 1, 1, 1), nhwc)[0] == "binarize_nhwc_kernel"
+    assert kernel_names((1, 32, 30, 6, 6, 3, 3, 1, 1, 1, 1), nhwc)[0] == "binarize_generic_kernel"
+    # the switch that forces the XNOR/popcount kernel (used to profile the two side by side)
+    monkeypatch.setenv("XNOR_NN_HIP_CONV", "valu")
+    assert kernel_names((256,) + conv4)[1] == "conv_xnor_popc_kernel<XW=12,Q=16>"
