@@ -360,6 +360,41 @@ def main():
         "device": {"name": props.name, "cus": cus, "clock_ghz": clk_hz / 1e9},
     }
     conv.close()
+    if not args.no_cold:
+        # What the memory system gives a kernel that only reads (xnor_nn_hip_plain_read: 16
+        # bytes per lane and load, nothing kept), for context beside the 8 TB/s the fractions
+        # are priced against: 1 GiB (four times the Infinity Cache: HBM), and this workload's
+        # own input re-read in place (cache-resident where it fits, as in the warm steps).
+        lib = capi.load()
+
+        def plain_read_us(tensor, passes=10):
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+            nbytes = tensor.numel() * tensor.element_size()
+            with torch.cuda.stream(stream):
+                for timed in (False, True):
+                    if timed:
+                        marks[0].record(stream)
+                    for _ in range(passes):
+                        if lib.xnor_nn_hip_plain_read(tensor.data_ptr(), nbytes,
+                                                      stream.cuda_stream) != capi.SUCCESS:
+                            sys.exit("xnor_nn_hip_plain_read failed")
+                    if timed:
+                        marks[1].record(stream)
+                    torch.cuda.synchronize()
+            return 1e3 * marks[0].elapsed_time(marks[1]) / passes
+
+        big = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        torch.cuda.synchronize()
+        big_us = plain_read_us(big)
+        del big
+        own_us = plain_read_us(xt)
+        result["roofline_binarize"]["plain_read"] = {
+            "of_1gib": {"duration_us": big_us, "achieved": (1 << 30) / (big_us * 1e-6) / 1e9,
+                        "frac": (1 << 30) / (big_us * 1e-6) / 1e9 / HBM_PEAK_GBS},
+            "of_this_input": {"bytes": xt.numel() * 4, "duration_us": own_us,
+                              "achieved": xt.numel() * 4 / (own_us * 1e-6) / 1e9},
+            "unit": "GB/s",
+            "how": "xnor_nn_hip_plain_read, 10 back-to-back passes between two events"}
     if args.copy_calibration_mib:
         n = args.copy_calibration_mib * (1 << 20) // 4
         src_buf = torch.ones(n, dtype=torch.float32, device=dev)

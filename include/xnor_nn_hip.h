@@ -112,6 +112,13 @@ int xnor_nn_hip_kernel_times(const xnor_nn_convolution_t *c, int stage, float *m
  * The reference's counterpart is its CPUID probe (reference src/utils/cpuid.hpp:119-168). */
 xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz);
 
+/* Calibration for benchmarks, no counterpart in the reference: enqueues on `stream` (a
+ * hipStream_t) one kernel that reads `bytes` (rounded down to 16) of device memory once, 16
+ * bytes per lane and load, and keeps nothing.  Its duration beside the binarize kernel's on
+ * the same bytes shows what the memory system, not the kernel, costs: the stages of this
+ * library that stream the input are priced against the HBM peak, which no reader reaches. */
+xnor_nn_status_t xnor_nn_hip_plain_read(const void *device_buffer, size_t bytes, void *stream);
+
 /* xnor_nn_binarize_weights_float (reference src/binarize_weights_float.cpp:3-25) for callers
  * that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  `from` and `to`

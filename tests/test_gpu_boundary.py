@@ -371,3 +371,19 @@ def test_verbose_lines_name_the_kernels(gpu, conv_kind):
         assert "box_filter_kernel" in execs[2]
         assert execs[3] == "xnor_nn exec forward: " + conv_name
     assert len(execs) == 4
+
+
+def test_plain_read_calibration_kernel(gpu):
+    """xnor_nn_hip_plain_read: runs on device memory of any size from one 16-byte piece up
+    (ragged ends included) and refuses what it cannot read."""
+    import torch
+    lib = capi.load()
+    for n in (4, 1000, 1 << 20, (1 << 22) + 5):
+        t = torch.ones(n, dtype=torch.float32, device=gpu)
+        assert lib.xnor_nn_hip_plain_read(t.data_ptr(), n * 4, None) == capi.SUCCESS
+    torch.cuda.synchronize()
+    host = np.ones(64, np.float32)
+    assert lib.xnor_nn_hip_plain_read(host.ctypes.data, host.nbytes, None) == capi.ERROR_INVALID_INPUT
+    assert lib.xnor_nn_hip_plain_read(None, 64, None) == capi.ERROR_INVALID_INPUT
+    assert lib.xnor_nn_hip_plain_read(t.data_ptr(), 8, None) == capi.ERROR_INVALID_INPUT
+    assert lib.xnor_nn_hip_plain_read(t.data_ptr() + 4, 64, None) == capi.ERROR_INVALID_INPUT

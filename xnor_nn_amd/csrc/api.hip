@@ -742,6 +742,15 @@ xnor_nn_status_t xnor_nn_hip_forward_popcount(const xnor_nn_convolution_t *c,
     return run_convolution(c, res, popc, true);
 }
 
+xnor_nn_status_t xnor_nn_hip_plain_read(const void *device_buffer, size_t bytes,
+        void *stream) {
+    if (device_buffer == nullptr || bytes < 16 || ((size_t)device_buffer & 15) != 0
+            || !on_device(device_buffer))
+        return xnor_nn_error_invalid_input;
+    return launch_plain_read(device_buffer, bytes, static_cast<hipStream_t>(stream))
+            == hipSuccess ? xnor_nn_success : xnor_nn_error_memory;
+}
+
 xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz) {
     int dev = 0, cus = 0, khz = 0;
     if (hipGetDevice(&dev) != hipSuccess

@@ -16,6 +16,7 @@ namespace {
 constexpr int TILE = 64;       // pixels per workgroup = lanes per wave
 constexpr int MAX_WAVES = 12;  // waves per workgroup
 constexpr int TURN_ROW = 36;   // floats per pixel row of the NHWC turn-around buffer (32 + 4)
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t fbits(float v) { return __float_as_uint(v); }
 
@@ -323,6 +324,22 @@ void box_filter_kernel(const float *__restrict__ a, float *__restrict__ k,
     k[p] = acc;
 }
 
+// Calibration only: reads a buffer once, 16 bytes per lane and load, four loads in flight per
+// lane, and keeps nothing.  What this takes is what the memory system allows a kernel that
+// does no work at all on the same bytes.
+__global__ __launch_bounds__(256)
+void plain_read_kernel(const v4u *__restrict__ x, const size_t n16) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    v4u acc = {0u, 0u, 0u, 0u};
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const v4u v0 = x[i], v1 = x[i + stride], v2 = x[i + 2 * stride], v3 = x[i + 3 * stride];
+        acc ^= v0 ^ v1 ^ v2 ^ v3;
+    }
+    for (; i < n16; i += stride) acc ^= x[i];
+    asm volatile("" : : "v"(acc)); // the loads have a use
+}
+
 template <bool NHWC, bool WRITE_BITS, bool WRITE_A>
 void launch_tiled(const Geometry &g, const float *x, uint32_t *bits, float *a, hipStream_t s,
         const KernelEvents &ev) {
@@ -430,6 +447,13 @@ hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStrea
         hipLaunchKernelGGL((binarize_generic_kernel<false, true>), dim3(blocks), dim3(256),
                 0, s, x, nullptr, a, g, inv_ic);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_plain_read(const void *buf, size_t bytes, hipStream_t s,
+        const KernelEvents &ev) {
+    launch_kernel(plain_read_kernel, dim3(2048), dim3(256), 0, s, ev,
+            static_cast<const v4u *>(buf), bytes / 16);
     return hipGetLastError();
 }
 

@@ -133,6 +133,9 @@ hipError_t launch_binarize_data(const Geometry &g, const float *x, uint32_t *bit
         float *a_or_null, hipStream_t s, const KernelEvents &ev = KernelEvents{});
 hipError_t launch_mean_abs(const Geometry &g, const float *x, float *a, hipStream_t s);
 hipError_t launch_box_filter(const Geometry &g, const float *a, float *k, hipStream_t s);
+// calibration: one pass of plain 16-byte reads over bytes / 16 * 16 bytes of device memory
+hipError_t launch_plain_read(const void *buf, size_t bytes, hipStream_t s,
+        const KernelEvents &ev = KernelEvents{});
 hipError_t launch_binarize_weights(const Geometry &g, const float *w, uint32_t *bits,
         float *alpha, int32_t *opc, hipStream_t s);
 hipError_t launch_convolution(const Geometry &g, const uint32_t *xbits,
