@@ -395,6 +395,35 @@ def main():
                               "achieved": xt.numel() * 4 / (own_us * 1e-6) / 1e9},
             "unit": "GB/s",
             "how": "xnor_nn_hip_plain_read, 10 back-to-back passes between two events"}
+    if not args.no_cold and on_mfma:
+        # What the matrix pipes give a kernel that only multiplies (xnor_nn_hip_mfma_only:
+        # register-resident pseudo-random +-1 operands, two workgroups per compute unit like
+        # the convolution, no operand traffic): the practical ceiling beside the published
+        # peak, which assumes the full clock.  As long a launch as the convolution takes, and
+        # a long one (the clock settles over milliseconds).
+        ops_per_wave_iter = 8 * 131072
+        rates = {}
+        for label, iters in (("short", 100), ("long", 20000)):
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+            reps = 20 if label == "short" else 1
+            with torch.cuda.stream(stream):
+                for timed in (False, True):
+                    if timed:
+                        marks[0].record(stream)
+                    for _ in range(reps):
+                        if lib.xnor_nn_hip_mfma_only(2 * cus, iters,
+                                                     stream.cuda_stream) != capi.SUCCESS:
+                            sys.exit("xnor_nn_hip_mfma_only failed")
+                    if timed:
+                        marks[1].record(stream)
+                    torch.cuda.synchronize()
+            us = 1e3 * marks[0].elapsed_time(marks[1]) / reps
+            tops = 2 * cus * 4 * iters * ops_per_wave_iter / (us * 1e-6) / 1e12
+            rates[label] = {"duration_us": us, "achieved": tops, "frac": tops / conv_peak}
+        result["roofline"]["matrix_instructions_only"] = dict(
+            rates, unit="TFLOP/s",
+            how="xnor_nn_hip_mfma_only, 2 workgroups per CU; short: 800 instructions per "
+                "wave, 20 launches back to back; long: 160000 per wave, one launch")
     if args.copy_calibration_mib:
         n = args.copy_calibration_mib * (1 << 20) // 4
         src_buf = torch.ones(n, dtype=torch.float32, device=dev)

@@ -119,6 +119,15 @@ xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz);
  * library that stream the input are priced against the HBM peak, which no reader reaches. */
 xnor_nn_status_t xnor_nn_hip_plain_read(const void *device_buffer, size_t bytes, void *stream);
 
+/* Calibration for benchmarks, no counterpart in the reference: enqueues one kernel of
+ * `workgroups` workgroups of four waves in which every wave issues 8 * iterations of the
+ * convolution kernel's matrix instruction (FP4 32x32x64 = 131072 operations each) on
+ * pseudo-random +-1 operands that stay in registers.  Its rate is what the matrix pipes
+ * deliver on such data with no operand traffic at all, under the chip's own clock management:
+ * the practical ceiling beside the published peak the convolution is priced against. */
+#define XNOR_NN_HIP_MFMA_ONLY_OPS_PER_WAVE_ITERATION (8 * 131072LL)
+xnor_nn_status_t xnor_nn_hip_mfma_only(int workgroups, int iterations, void *stream);
+
 /* xnor_nn_binarize_weights_float (reference src/binarize_weights_float.cpp:3-25) for callers
  * that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  `from` and `to`

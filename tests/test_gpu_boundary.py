@@ -387,3 +387,14 @@ def test_plain_read_calibration_kernel(gpu):
     assert lib.xnor_nn_hip_plain_read(None, 64, None) == capi.ERROR_INVALID_INPUT
     assert lib.xnor_nn_hip_plain_read(t.data_ptr(), 8, None) == capi.ERROR_INVALID_INPUT
     assert lib.xnor_nn_hip_plain_read(t.data_ptr() + 4, 64, None) == capi.ERROR_INVALID_INPUT
+
+
+def test_matrix_instruction_calibration_kernel(gpu):
+    """xnor_nn_hip_mfma_only runs (it touches no memory) and checks its two counts."""
+    import torch
+    lib = capi.load()
+    assert lib.xnor_nn_hip_mfma_only(8, 3, None) == capi.SUCCESS
+    assert lib.xnor_nn_hip_mfma_only(512, 50, None) == capi.SUCCESS
+    torch.cuda.synchronize()
+    assert lib.xnor_nn_hip_mfma_only(0, 3, None) == capi.ERROR_INVALID_INPUT
+    assert lib.xnor_nn_hip_mfma_only(8, 0, None) == capi.ERROR_INVALID_INPUT

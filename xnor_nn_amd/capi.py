@@ -65,6 +65,7 @@ HIP_SYMBOLS = {
     "xnor_nn_hip_set_stream": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_void_p]),
     "xnor_nn_hip_set_stage_fusion": (C.c_int, [C.POINTER(ConvolutionDesc), C.c_int]),
     "xnor_nn_hip_plain_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "xnor_nn_hip_mfma_only": (C.c_int, [C.c_int, C.c_int, C.c_void_p]),
     "xnor_nn_hip_synchronize": (C.c_int, [C.POINTER(ConvolutionDesc)]),
     "xnor_nn_hip_export_bin_src": (C.c_int, [C.POINTER(ConvolutionDesc), C.POINTER(C.c_void_p), C.c_void_p, C.c_size_t]),
     "xnor_nn_hip_export_bin_weights": (C.c_int, [C.POINTER(ConvolutionDesc), C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_size_t]),

@@ -751,6 +751,13 @@ xnor_nn_status_t xnor_nn_hip_plain_read(const void *device_buffer, size_t bytes,
             == hipSuccess ? xnor_nn_success : xnor_nn_error_memory;
 }
 
+xnor_nn_status_t xnor_nn_hip_mfma_only(int workgroups, int iterations, void *stream) {
+    if (workgroups < 1 || workgroups > (1 << 20) || iterations < 1 || iterations > (1 << 20))
+        return xnor_nn_error_invalid_input;
+    return launch_mfma_only(workgroups, iterations, static_cast<hipStream_t>(stream))
+            == hipSuccess ? xnor_nn_success : xnor_nn_error_memory;
+}
+
 xnor_nn_status_t xnor_nn_hip_device_info(int *compute_units, int *clock_khz) {
     int dev = 0, cus = 0, khz = 0;
     if (hipGetDevice(&dev) != hipSuccess

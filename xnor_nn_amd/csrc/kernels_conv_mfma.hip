@@ -804,6 +804,50 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     }
 }
 
+// Calibration only: the matrix instruction of the convolution kernel and nothing else.  Every
+// wave multiplies pseudo-random +-1 fragments (the FP4 codes 0x2 and 0xA) that never leave
+// its registers into eight independent accumulator blocks, `iterations` times.  What this
+// reaches is what the matrix pipes deliver on this data under the chip's power management,
+// with no operand traffic at all.
+__global__ __launch_bounds__(256, 2)
+void mfma_only_kernel(const int iterations) {
+    auto signs = [](uint32_t h) { // eight FP4 codes, sign bits from h
+        h *= 0x9E3779B1u;
+        h ^= h >> 15;
+        uint32_t spread = 0;
+#pragma unroll
+        for (int n = 0; n < 8; n++) spread |= ((h >> n) & 1u) << (4 * n + 3);
+        return (int)(0x22222222u | spread);
+    };
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    v4i a[2], b[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+        a[i] = v4i{signs(id * 24u + i * 4u), signs(id * 24u + i * 4u + 1), signs(id * 24u + i * 4u + 2),
+                   signs(id * 24u + i * 4u + 3)};
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        b[i] = v4i{signs(id * 24u + 8u + i * 4u), signs(id * 24u + 9u + i * 4u),
+                   signs(id * 24u + 10u + i * 4u), signs(id * 24u + 11u + i * 4u)};
+    v16f acc[2][4];
+#pragma unroll
+    for (int os = 0; os < 2; os++)
+#pragma unroll
+        for (int ps = 0; ps < 4; ps++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[os][ps][i] = 0.f;
+    for (int it = 0; it < iterations; it++) {
+#pragma unroll
+        for (int os = 0; os < 2; os++)
+#pragma unroll
+            for (int ps = 0; ps < 4; ps++) acc[os][ps] = mfma_fp4(a[os], b[ps], acc[os][ps]);
+    }
+#pragma unroll
+    for (int os = 0; os < 2; os++)
+#pragma unroll
+        for (int ps = 0; ps < 4; ps++) asm volatile("" : : "v"(acc[os][ps]));
+}
+
 // One thread per dword of the fragment layout [OC/32][tap][KS][lane][4 dwords]:
 // lane l of a fragment holds filter (l % 32) and channels (l / 32) * 32 .. +31 of the step,
 // eight channels per dword, low nibble first.  Channels >= IC and filters >= OC are FP4 zero.
@@ -1141,6 +1185,11 @@ void mfma_plan(Geometry &g) {
             g.mfma_lds = (uint32_t)lds;
         }
     }
+}
+
+hipError_t launch_mfma_only(int workgroups, int iterations, hipStream_t s) {
+    hipLaunchKernelGGL(mfma_only_kernel, dim3((unsigned)workgroups), dim3(256), 0, s, iterations);
+    return hipGetLastError();
 }
 
 hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *frag,

@@ -162,6 +162,9 @@ hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k,
         float *dst, int32_t *popc_or_null, const float *a_or_null, float *k_out,
         hipStream_t s, const KernelEvents &ev = KernelEvents{});
+// calibration: `workgroups` x 4 waves, each issuing 8 * iterations FP4 matrix instructions
+// (32x32x64) on register-resident +-1 operands
+hipError_t launch_mfma_only(int workgroups, int iterations, hipStream_t s);
 const char *convolution_kernel_name(const Geometry &g);
 const char *binarize_kernel_name(const Geometry &g);
 
