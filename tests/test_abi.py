@@ -255,8 +255,9 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
         == "conv_mfma_fp4_kernel<KS=3,PS=4,PAIR>"
     assert kernel_names((64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
         == "conv_mfma_fp4_kernel<KS=4,PS=4>"
+    # 98 blocks for 32 slots per XCD and filter chunk: 2 tiles of four, 30 of three
     assert kernel_names((32, 512, 512, 28, 28, 3, 3, 1, 1, 1, 1))[1] \
-        == "conv_mfma_fp4_kernel<KS=8,PS=4>"
+        == "conv_mfma_fp4_kernel<KS=8,PS=4+3>"
     # more than 1024 channels: channel parts; more than 4096: no matrix cores
     assert re.fullmatch(r"conv_mfma_fp4_kernel<KS=1[26],PS=\d,PARTS=\d>",
                         kernel_names((2, 64, 2048, 8, 8, 3, 3, 1, 1, 1, 1))[1])

@@ -658,7 +658,7 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
     """Fifteen seconds of seeded random problems larger than the ones above (channel counts
     around the 32/64/1024 boundaries up to 2048, kernels 1..9, strides 1..4, paddings 0..4,
     images up to 43 x 43, every layout combination, inputs with exact zeros of both signs;
-    every third problem with the two-tile-size launch forced on, every fourth with streaming
+    every third problem with a two-tile-size launch forced on (four and two, four and three), every fourth with streaming
     output stores): dst and the raw popcounts against the oracle, bit for bit, stopping at
     the first mismatch."""
     import time
@@ -695,7 +695,7 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
         ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
         want = oracle.forward(oracle_shape(oracle, d, fmts), xs, ws)
         # launch options that the library otherwise picks by problem size
-        forced = {"XNOR_NN_HIP_MFMA_MIX": "1" if n % 3 == 2 else None,
+        forced = {"XNOR_NN_HIP_MFMA_MIX": "1" if n % 6 == 2 else "3" if n % 6 == 5 else None,
                   "XNOR_NN_HIP_STREAM_DST": "1" if n % 4 == 3 else None}
         for key, value in forced.items():
             if value is None:
@@ -740,12 +740,16 @@ def test_streaming_output_stores(oracle, gpu, monkeypatch, fmts):
     ((5, 64, 64, 28, 28, 3, 3, 2, 2, 1, 1), (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC)),
     ((2, 512, 200, 14, 14, 3, 3, 1, 1, 1, 1), NCHW),                     # 8 steps per tap
     ((1, 33, 32, 5, 5, 3, 3, 1, 1, 1, 1), NCHW),                         # a single pixel block
+    ((3, 512, 512, 14, 14, 3, 3, 1, 1, 1, 1), NCHW),                     # two filter chunks
+    ((6, 64, 600, 11, 9, 3, 3, 1, 1, 1, 1), (capi.FMT_NCHW, capi.FMT_HWIO, capi.FMT_NHWC)),
 ], ids=lambda v: shapes.shape_id(v) if len(v) == 11 else "fmt%d%d%d" % v)
-def test_two_tile_sizes_in_one_launch(oracle, monkeypatch, t, fmts):
+@pytest.mark.parametrize("small", [2, 3])
+def test_two_tile_sizes_in_one_launch(oracle, monkeypatch, t, fmts, small):
     """The matrix-core kernel with four-block tiles for the first workgroups of an XCD and
-    two-block tiles for the rest (chosen by size at init; the full-size conv4 workload above
-    takes it), forced on for problems whose XCD ranges end raggedly or hold no big tile."""
-    monkeypatch.setenv("XNOR_NN_HIP_MFMA_MIX", "1")
+    two- or three-block tiles for the rest (chosen by size at init; the full-size conv4 and
+    VGG workloads above take one each), forced on for problems whose XCD ranges end raggedly,
+    hold no big tile, or have several filter chunks."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_MIX", "1" if small == 2 else "3")
     d = shapes.as_dims(t)
     x = synth.normal(151, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
         d["mb"], d["ic"], d["ih"], d["iw"])
@@ -753,5 +757,5 @@ def test_two_tile_sizes_in_one_launch(oracle, monkeypatch, t, fmts):
     w = synth.normal(152, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
         d["oc"], d["ic"], d["kh"], d["kw"])
     name = make(d, w, fmts).kernel_name(0)
-    assert "PS=4+2" in name, name
+    assert "PS=4+%d" % small in name, name
     run_and_compare(oracle, d, x, w, fmts)

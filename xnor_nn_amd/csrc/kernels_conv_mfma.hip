@@ -761,9 +761,10 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
 // range of tiles, so the input rows two neighbouring tiles share and the output cache lines
 // they both write into meet in one L2.  A unit is a (tile, filter chunk) pair.
 //
-// PSB > 0, two tile sizes (one filter chunk only): XCD x owns the pixel blocks
-// [x * blocks_per_xcd, (x+1) * blocks_per_xcd); its first big_per_xcd workgroups take PS
-// blocks each, the following ones PSB blocks each.  The hardware starts workgroups in the
+// PSB > 0, two tile sizes: XCD x owns the pixel blocks
+// [x * blocks_per_xcd, (x+1) * blocks_per_xcd); its first big_per_xcd tiles have PS blocks
+// each, the following ones PSB blocks each, and workgroup n of the XCD takes tile
+// n / oc_chunks with filter chunk n % oc_chunks.  The hardware starts workgroups in the
 // order of their index and the matrix pipe serves the older wave of a SIMD first, so on a
 // compute unit that holds two workgroups the one with the small tile is the one that
 // finishes last: its epilogue, the only one nothing overlaps, is the short one.
@@ -788,18 +789,20 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     } else {
         const uint32_t first = xcd * blocks_per_xcd; // pixel blocks of this XCD: [first, last)
         const uint32_t p_limit = min((first + blocks_per_xcd) * 32u, g.npix_out);
-        if (nth < big_per_xcd) {
-            const uint32_t p_first = (first + nth * PS) * 32u;
+        const uint32_t tile = oc_chunks == 1 ? nth : nth / oc_chunks;
+        const int chunk = nth - tile * oc_chunks;
+        if (tile < big_per_xcd) {
+            const uint32_t p_first = (first + tile * PS) * 32u;
             if (p_first >= p_limit) return;
             conv_tile<KS, PS, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g,
                     max_rows, div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, p_first,
-                    p_limit, 0);
+                    p_limit, chunk);
         } else {
-            const uint32_t p_first = (first + big_per_xcd * PS + (nth - big_per_xcd) * PSB) * 32u;
+            const uint32_t p_first = (first + big_per_xcd * PS + (tile - big_per_xcd) * PSB) * 32u;
             if (p_first >= p_limit) return;
             conv_tile<KS, PSB, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g,
                     max_rows, div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, p_first,
-                    p_limit, 0);
+                    p_limit, chunk);
         }
     }
 }
@@ -1038,7 +1041,7 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         blocks = g.mfma_blocks_per_xcd;
         big = g.mfma_big_per_xcd;
         const uint32_t rest = blocks > big * PS ? blocks - big * PS : 0;
-        per_xcd = big + (rest + PSB - 1) / PSB;
+        per_xcd = (big + (rest + PSB - 1) / PSB) * chunks;
     }
     const dim3 grid(per_xcd * 8), block(256);
     const int rows = g.mfma_rows;
@@ -1091,10 +1094,14 @@ template <int KS, bool PAIR = false>
 hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
-    if (g.mfma_ps_small > 0) { // four blocks for the first workgroup of a CU, two for the second
-        if constexpr (KS < 16 && !(PAIR && KS >= 5))
+    if (g.mfma_ps_small > 0) { // two tile sizes: four blocks, and two or three
+        if constexpr (KS < 16 && !(PAIR && KS >= 5)) {
+            if (g.mfma_ps_small == 3)
+                return launch_mfma<KS, 4, PAIR, false, 3>(g, xbits, wfrag, alpha, k, dst, popc,
+                        a_or_null, k_out, s, ev);
             return launch_mfma<KS, 4, PAIR, false, 2>(g, xbits, wfrag, alpha, k, dst, popc,
                     a_or_null, k_out, s, ev);
+        }
         return hipErrorInvalidValue;
     }
     switch (g.mfma_ps) {
@@ -1162,25 +1169,42 @@ void mfma_plan(Geometry &g) {
     g.mfma_wbytes = (uint32_t)mfma_weight_bytes(g);
     // Two tile sizes in one launch (see the kernel): worth it when every compute unit gets
     // more than four and at most six pixel blocks, i.e. when equal tiles would give it two
-    // workgroups of three that finish together.  Needs one filter chunk, the four-block
-    // variant, and room for two workgroups in a CU's LDS.  XNOR_NN_HIP_MFMA_MIX=0|1 overrides
-    // the size rule (for measurements), a forced tile size switches it off.
+    // workgroups of three that finish together.  Needs the four-block variant and room for
+    // two workgroups in a CU's LDS.  XNOR_NN_HIP_MFMA_MIX=0|1|3 overrides the size rules (off,
+    // four and two, four and three; for measurements), a forced tile size switches them off.
     const uint32_t blocks = (g.npix_out + 31) / 32, blocks_per_xcd = (blocks + 7) / 8;
     const uint32_t cus_per_xcd = (uint32_t)(g.cus + 7) / 8;
-    bool mix = blocks_per_xcd > 4 * cus_per_xcd && blocks_per_xcd <= 6 * cus_per_xcd;
-    if (const char *e = getenv("XNOR_NN_HIP_MFMA_MIX")) mix = e[0] == '1';
-    if (getenv("XNOR_NN_HIP_MFMA_PS") || g.oc > NT || g.mfma_parts > 1 || g.mfma_steps >= 16
+    // The same in filter chunks: `slots` workgroups per XCD and chunk when every CU holds two.
+    const uint32_t chunks = (uint32_t)(g.oc + NT - 1) / NT;
+    const uint32_t slots = 2 * cus_per_xcd / chunks;
+    bool mix = chunks == 1 && blocks_per_xcd > 4 * cus_per_xcd && blocks_per_xcd <= 6 * cus_per_xcd;
+    // Between three and four blocks per slot, equal tiles of four leave slots empty and tiles
+    // of three need a second round for the last few: blocks - 3 * slots tiles of four and
+    // tiles of three for the rest fill every slot exactly once (VGG 512, MB 32: 98 blocks
+    // and 32 slots per XCD and chunk: 2 tiles of four, 30 of three).
+    bool fill = slots > 0 && blocks_per_xcd > 3 * slots && blocks_per_xcd < 4 * slots;
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_MIX")) {
+        mix = e[0] == '1';
+        fill = e[0] == '3';
+    }
+    if (getenv("XNOR_NN_HIP_MFMA_PS") || g.mfma_parts > 1 || g.mfma_steps >= 16
             || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4))
-        mix = false;
-    if (mix) {
+        mix = fill = false;
+    if (mix || fill) {
         const int rows = max_tile_rows(g, 32 * 4, 32);
         const size_t lds = lds_bytes_for(g, (size_t)rows, 4);
         if (lds <= (size_t)LDS_TWO_PER_CU) {
             g.mfma_ps = 4;
-            g.mfma_ps_small = 2;
             g.mfma_blocks_per_xcd = blocks_per_xcd;
-            const uint32_t fit = blocks_per_xcd / 4; // whole four-block tiles in an XCD's range
-            g.mfma_big_per_xcd = fit < cus_per_xcd ? fit : cus_per_xcd;
+            if (mix) {
+                g.mfma_ps_small = 2;
+                const uint32_t fit = blocks_per_xcd / 4; // whole four-block tiles in the range
+                g.mfma_big_per_xcd = fit < cus_per_xcd ? fit : cus_per_xcd;
+            } else {
+                g.mfma_ps_small = 3;
+                g.mfma_big_per_xcd = blocks_per_xcd > 3 * slots ? blocks_per_xcd - 3 * slots : 0;
+                if (g.mfma_big_per_xcd > blocks_per_xcd / 4) g.mfma_big_per_xcd = blocks_per_xcd / 4;
+            }
             g.mfma_rows = rows;
             g.mfma_lds = (uint32_t)lds;
         }
