@@ -11,10 +11,19 @@ vector memory (loads and stores, which return in order and share vmcnt) and LDS 
 writes; LDS operations complete in order among themselves, so after lgkmcnt(N) all but the
 newest N of them are done whatever scalar memory loads share the counter).
 
+What is tracked are the loads the source issues by hand: the instructions between the
+compiler's ";;#ASMSTART" and ";;#ASMEND" markers.  Loads that the compiler issues itself
+(builtins, ordinary pointer reads) are covered by its own wait insertion, which knows their
+destinations; they are not tracked, but they are counted, because every operation in a queue
+ages the ones ahead of it.  (Tracking them as well reports paths that cannot be taken: the
+compiler guards a load and the wait that covers it with the same lane mask, and a walk that
+knows nothing about branch conditions takes the load and skips the wait.  The same goes for a
+kernel made of two inlined tile bodies, where falling from the first body into the second is
+a path the hardware never takes.)  Every kernel is walked from its first instruction, so a
+kernel with several tile bodies, or a loop over tiles around one body, is covered whole.
+
 Only the matrix-core kernel is walked.  The streaming kernels of stages 1 and 2 issue their
-buffer loads through compiler builtins, so the compiler's own wait insertion covers them; a
-walk that knows nothing about branch conditions reports paths there that cannot be taken
-(a wave that skips its turn in the ordered hand-over of the running sum)."""
+buffer loads through compiler builtins only."""
 import os
 import re
 import subprocess
@@ -26,6 +35,8 @@ from xnor_nn_amd import build
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "xnor_nn_amd", "csrc")
 VM_MAX, LGKM_MAX = 64, 16
+ASM_BEGIN, ASM_END = "#ASMSTART", "#ASMEND"
+EXPECTED_VARIANTS = 132  # kernels the matrix-core file instantiates
 
 
 def vgprs(token):
@@ -41,9 +52,20 @@ def parse(body):
     """One tuple per line: (kind, registers touched, vector-memory destination, LDS
     destination, (vmcnt, lgkmcnt), branch target); a destination of frozenset() is an
     operation that counts without writing a register (a store, an LDS write)."""
-    label_at = {l[:-1]: i for i, l in enumerate(body) if l.startswith(".LBB")}
+    body = [l for l in body]
+    label_at, n = {}, 0
+    for l in body:  # index of every label among the parsed entries (markers produce none)
+        if l in (ASM_BEGIN, ASM_END):
+            continue
+        if l.startswith(".LBB"):
+            label_at[l[:-1]] = n
+        n += 1
     out = []
+    by_hand = False
     for line in body:
+        if line in (ASM_BEGIN, ASM_END):
+            by_hand = line == ASM_BEGIN
+            continue
         if line.startswith(".LBB"):
             out.append(("label", None, None, None, None, None))
             continue
@@ -74,8 +96,16 @@ def parse(body):
             elif op.startswith("ds_"):
                 ldst = frozenset() if re.match(r"ds_(write|add|sub|min|max|and|or|xor)", op) \
                     and "_rtn" not in op else vgprs(ops[0])
+            if not by_hand:  # the compiler's own: counted, not tracked
+                vdst = frozenset() if vdst is not None else None
+                ldst = frozenset() if ldst is not None else None
             out.append(("vector", touched, vdst, ldst, None, None))
     return out
+
+
+def instructions(body):
+    """The lines of a body that parse() turns into entries, in the same order."""
+    return [l for l in body if l not in (ASM_BEGIN, ASM_END)]
 
 
 def hazards_of(body, first=0):
@@ -89,6 +119,7 @@ def hazards_of(body, first=0):
     completed.  Where paths meet (labels), a register keeps the smaller of its ages: the walk
     is a fixed-point iteration over the control flow graph, conservative where paths differ."""
     code = parse(body)
+    body = instructions(body)
     at_label, work, bad = {}, [(first, {}, {})], set()
 
     def issue(ages, dst, limit):
@@ -154,38 +185,99 @@ def kernels_of(isa, pattern):
     """(mangled name, instructions and labels) of every kernel whose symbol matches."""
     for st in [i for i, l in enumerate(isa) if re.match(pattern, l)]:
         end = next(i for i in range(st, len(isa)) if ".end_amdhsa_kernel" in isa[i])
-        body = [l.strip().split(";")[0].rstrip() for l in isa[st:end]]
-        yield isa[st], [l for l in body if l and (not l.startswith(".") or l.startswith(".LBB"))]
+        body = []
+        for l in isa[st:end]:
+            l = l.strip()
+            if l.startswith(";;" + ASM_BEGIN) or l.startswith(";;" + ASM_END):
+                body.append(l[2:].split()[0])
+                continue
+            l = l.split(";")[0].rstrip()
+            if l and (not l.startswith(".") or l.startswith(".LBB")):
+                body.append(l)
+        yield isa[st], body
+
+
+def by_hand(*lines):
+    """The lines as the compiler prints an inline-asm statement."""
+    return [ASM_BEGIN] + list(lines) + [ASM_END]
 
 
 def test_no_register_is_touched_while_its_load_is_in_flight(tmp_path):
     """Every variant of the matrix-core kernel that the library holds (all of them can be
-    launched), from its first hand-issued fragment load to the end."""
+    launched), from its first instruction to the end."""
     isa = compile_to_isa(tmp_path, "kernels_conv_mfma")
     checked = 0
-    for name, body in kernels_of(isa, r"^_ZN\S*conv_mfma_fp4_kernel\S*:"):
-        first = next((i for i, l in enumerate(body) if l.startswith("buffer_load_dwordx4")),
-                     None)
-        assert first is not None, "no fragment loads found in " + name
-        bad = hazards_of(body, first)
+    for name, body in kernels_of(isa, r"^_ZN\S*conv_mfma_fp4\S*kernel\S*:"):
+        lines = instructions(body)
+        code = parse(body)
+        tracked = sum(1 for c in code if c[0] == "vector" and (c[2] or c[3]))
+        assert tracked >= 4, "no hand-issued loads found in " + name
+        assert len(code) == len(lines)
+        bad = hazards_of(body)
         assert not bad, "%s: %d instructions touch a register whose load is in flight, " \
             "first: %s" % (name[:90], len(bad), bad[0][1])
         checked += 1
-    assert checked >= 90
+    assert checked >= EXPECTED_VARIANTS, checked
 
 
 def test_the_walker_sees_a_planted_hazard():
     """The checker itself: a register read one instruction before the wait that covers its
     load, for a vector memory load and for an LDS read, and the same code with the wait in
     place."""
-    ok = ["buffer_load_dwordx4 v[4:7], v1, s[0:3], 0 offen", "ds_read_b128 v[8:11], v2",
-          "s_waitcnt vmcnt(0) lgkmcnt(0)", "v_add_u32_e32 v3, v4, v8", "s_endpgm"]
+    load = "buffer_load_dwordx4 v[4:7], v1, s[0:3], 0 offen"
+    read = "ds_read_b128 v[8:11], v2"
+    use = "v_add_u32_e32 v3, v4, v8"
+    ok = by_hand(load) + by_hand(read) + ["s_waitcnt vmcnt(0) lgkmcnt(0)", use, "s_endpgm"]
     assert hazards_of(ok) == []
-    early_vm = [ok[0], ok[1], "s_waitcnt lgkmcnt(0)", ok[3], ok[4]]
-    assert [b[1] for b in hazards_of(early_vm)] == [ok[3]]
-    early_lds = [ok[0], ok[1], "s_waitcnt vmcnt(0)", ok[3], ok[4]]
-    assert [b[1] for b in hazards_of(early_lds)] == [ok[3]]
+    early_vm = by_hand(load) + by_hand(read) + ["s_waitcnt lgkmcnt(0)", use, "s_endpgm"]
+    assert [b[1] for b in hazards_of(early_vm)] == [use]
+    early_lds = by_hand(load) + by_hand(read) + ["s_waitcnt vmcnt(0)", use, "s_endpgm"]
+    assert [b[1] for b in hazards_of(early_lds)] == [use]
     # in-order return: with one operation allowed in flight the older of two is done
-    two = ["ds_read_b128 v[4:7], v2", "ds_read_b128 v[8:11], v2 offset:16",
-           "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v0, v4", "v_mov_b32_e32 v1, v8", "s_endpgm"]
+    two = by_hand("ds_read_b128 v[4:7], v2", "ds_read_b128 v[8:11], v2 offset:16") + [
+        "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v0, v4", "v_mov_b32_e32 v1, v8", "s_endpgm"]
     assert [b[1] for b in hazards_of(two)] == ["v_mov_b32_e32 v1, v8"]
+    # a wait inside the asm statement itself (wait, then start the next reads) is seen
+    fused = by_hand(read) + by_hand("s_waitcnt lgkmcnt(0)", "ds_read_b128 v[12:15], v2") + [
+        "v_mov_b32_e32 v0, v8", "v_mov_b32_e32 v1, v12", "s_endpgm"]
+    assert [b[1] for b in hazards_of(fused)] == ["v_mov_b32_e32 v1, v12"]
+
+
+def test_the_compilers_own_loads_are_counted_but_not_tracked():
+    """A load outside the asm markers is the compiler's: its destination is not followed
+    (the compiler waits for it itself), but it ages what is in flight ahead of it."""
+    load = "buffer_load_dwordx4 v[4:7], v1, s[0:3], 0 offen"
+    own = "global_load_dword v29, v[30:31], off"
+    # the compiler's load and its guarded wait: taking the load and skipping the wait is a
+    # path of the walk that the hardware never takes, and nothing is reported for it
+    guarded = [own, "s_and_saveexec_b64 s[4:5], vcc", "s_cbranch_execz .LBB0_2", ".LBB0_1:",
+               "s_waitcnt vmcnt(0)", "ds_write_b32 v2, v29", ".LBB0_2:", own, "s_endpgm"]
+    assert hazards_of(guarded) == []
+    # ... but one load by hand followed by one of the compiler's: vmcnt(1) covers the first
+    aged = by_hand(load) + [own, "s_waitcnt vmcnt(1)", "v_mov_b32_e32 v0, v4", "s_endpgm"]
+    assert hazards_of(aged) == []
+    not_aged = by_hand(load) + ["s_waitcnt vmcnt(1)", "v_mov_b32_e32 v0, v4", "s_endpgm"]
+    assert [b[1] for b in hazards_of(not_aged)] == ["v_mov_b32_e32 v0, v4"]
+
+
+def test_a_hazard_in_a_second_body_is_seen():
+    """A kernel of two inlined tile bodies, as the compiler lays out `if (big) body1 else
+    body2` with a uniform skip over the second body (s_mov_b64 sX, 0 / s_andn2_b64 vcc, exec,
+    sX / s_cbranch_vccnz): the first body is clean, the second touches a fragment register
+    ahead of its wait.  Both the entry branch and the fall-through reach the second body."""
+    load = "buffer_load_dwordx4 v[4:7], v1, s[0:3], 0 offen"
+    body1 = by_hand(load) + ["s_waitcnt vmcnt(0)", "v_mov_b32_e32 v0, v4"]
+    skip = ["s_mov_b64 s[0:1], 0", "s_andn2_b64 vcc, exec, s[0:1]", "s_cbranch_vccnz .LBB0_3"]
+    body2_bad = [".LBB0_2:"] + by_hand(load) + ["v_mov_b32_e32 v0, v5", "s_waitcnt vmcnt(0)"]
+    body2_ok = [".LBB0_2:"] + by_hand(load) + ["s_waitcnt vmcnt(0)", "v_mov_b32_e32 v0, v5"]
+    head = ["s_cmp_lt_u32 s8, s9", "s_cbranch_scc0 .LBB0_2"]
+    tail = [".LBB0_3:", "s_endpgm"]
+    assert [b[1] for b in hazards_of(head + body1 + skip + body2_bad + tail)] \
+        == ["v_mov_b32_e32 v0, v5"]
+    assert hazards_of(head + body1 + skip + body2_ok + tail) == []
+    # a loop over tiles around one body: a load left in flight at the back edge is seen at
+    # the top of the next round
+    loop = [".LBB0_1:", "v_mov_b32_e32 v0, v4"] + by_hand(load) + [
+        "s_cmp_lt_u32 s8, s9", "s_cbranch_scc1 .LBB0_1", "s_waitcnt vmcnt(0)", "s_endpgm"]
+    # (and so is the second load into registers whose first load has not arrived)
+    assert [b[1] for b in hazards_of(loop)] == ["v_mov_b32_e32 v0, v4", load]
