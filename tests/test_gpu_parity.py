@@ -658,8 +658,9 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
     """Fifteen seconds of seeded random problems larger than the ones above (channel counts
     around the 32/64/1024 boundaries up to 2048, kernels 1..9, strides 1..4, paddings 0..4,
     images up to 43 x 43, every layout combination, inputs with exact zeros of both signs;
-    every third problem with a two-tile-size launch forced on (four and two, four and three), every fourth with streaming
-    output stores): dst and the raw popcounts against the oracle, bit for bit, stopping at
+    every third problem with a two-tile-size launch forced on (four and two, four and three),
+    every third with persistent workgroups forced on (one to three per XCD, so that each walks
+    over many tiles), every fourth with streaming output stores): dst and the raw popcounts against the oracle, bit for bit, stopping at
     the first mismatch."""
     import time
     rng = np.random.default_rng(20251)
@@ -696,6 +697,7 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
         want = oracle.forward(oracle_shape(oracle, d, fmts), xs, ws)
         # launch options that the library otherwise picks by problem size
         forced = {"XNOR_NN_HIP_MFMA_MIX": "1" if n % 6 == 2 else "3" if n % 6 == 5 else None,
+                  "XNOR_NN_HIP_MFMA_PERSIST": str(1 + n % 3) if n % 6 in (0, 3) else None,
                   "XNOR_NN_HIP_STREAM_DST": "1" if n % 4 == 3 else None}
         for key, value in forced.items():
             if value is None:
@@ -759,3 +761,39 @@ def test_two_tile_sizes_in_one_launch(oracle, monkeypatch, t, fmts, small):
     name = make(d, w, fmts).kernel_name(0)
     assert "PS=4+%d" % small in name, name
     run_and_compare(oracle, d, x, w, fmts)
+
+
+@pytest.mark.parametrize("t,fmts", [
+    ((40, 384, 256, 13, 13, 3, 3, 1, 1, 1, 1), NCHW),                    # conv4: 212 blocks, 27 per XCD
+    ((7, 384, 256, 13, 13, 3, 3, 1, 1, 1, 1), NCHW),                     # fewer blocks than XCDs x 4
+    ((3, 96, 130, 27, 27, 5, 5, 1, 1, 2, 2), NCHW),                      # paired taps, ragged filters
+    ((5, 64, 64, 28, 28, 3, 3, 2, 2, 1, 1), (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC)),
+    ((2, 512, 200, 14, 14, 3, 3, 1, 1, 1, 1), NCHW),                     # 8 steps per tap
+    ((1, 33, 32, 5, 5, 3, 3, 1, 1, 1, 1), NCHW),                         # a single pixel block
+    ((3, 512, 512, 14, 14, 3, 3, 1, 1, 1, 1), NCHW),                     # two filter chunks
+    ((6, 64, 600, 11, 9, 3, 3, 1, 1, 1, 1), (capi.FMT_NCHW, capi.FMT_HWIO, capi.FMT_NHWC)),
+    ((4, 256, 40, 56, 56, 3, 3, 1, 1, 1, 1), NCHW),                      # ResNet rows, one wave with filters
+    ((9, 100, 70, 17, 23, 5, 3, 2, 1, 2, 1), NCHW),                      # strides, ragged everything
+], ids=lambda v: shapes.shape_id(v) if len(v) == 11 else "fmt%d%d%d" % v)
+@pytest.mark.parametrize("wgs", [1, 2, 3, 64])
+def test_persistent_workgroups(oracle, monkeypatch, t, fmts, wgs):
+    """The matrix-core kernel with workgroups that stay and walk over their tiles (chosen by
+    size at init when a workgroup slot gets six pixel blocks or more; the full-size ResNet and
+    conv2-shape workloads above take it), forced on here with `wgs` workgroups per XCD: with
+    one to three of them every workgroup walks over many tiles of both sizes, copies the next
+    tile's packed words into LDS while it multiplies, and meets XCD ranges that end raggedly;
+    with 64 most workgroups get one tile or none."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_PERSIST", str(wgs))
+    d = shapes.as_dims(t)
+    x = synth.normal(161, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::6] = 0.0
+    w = synth.normal(162, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    xs = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if fmts[0] == capi.FMT_NHWC else x
+    ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
+    name = make(d, ws, fmts).kernel_name(0)
+    chunks = (d["oc"] + 255) // 256
+    if wgs >= chunks:
+        assert name.startswith("conv_mfma_fp4_persistent_kernel"), name
+    run_and_compare(oracle, d, xs, ws, fmts)

@@ -84,9 +84,11 @@ __host__ __device__ inline void tile_span(const Geometry &g, uint32_t p_first, u
 __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c) {
     const v8i a8 = {a.x, a.y, a.z, a.w, 0, 0, 0, 0};
     const v8i b8 = {b.x, b.y, b.z, b.w, 0, 0, 0, 0};
-    // cbsz = blgp = 4: both operands FP4 (E2M1); scales 0x7f = 2^0
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, 0, 0x7f7f7f7f, 0,
-            0x7f7f7f7f);
+    // cbsz = blgp = 4: both operands FP4 (E2M1).  Scale operands of zero select the plain
+    // v_mfma_f32_32x32x64_f8f6f4, which multiplies the operands as they are; a scale of 2^0
+    // passed in registers gives the same products through v_mfma_scale_..., which costs a
+    // v_mfma_ld_scale_b32 and a scale register read per matrix instruction.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, 0, 0, 0, 0);
 }
 
 // Operand traffic is issued by hand.  Left to itself the compiler hoists the global loads of
@@ -184,6 +186,36 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
     return out;
 }
 
+// What a persistent workgroup carries from one tile to the next (conv_tile with PERSIST).
+// The packed input words of a tile (and mean|x| of its input pixels) are copied into one of two
+// LDS staging areas while the tile before it is multiplied, so that a tile's staging phase
+// reads LDS only and waits for no global load.
+struct TileTurn {
+    bool first;          // the workgroup's first tile: table, zero row, alphas are not in LDS yet
+    uint32_t parity;     // which staging area holds this tile's words
+    uint32_t next_first, next_end; // output pixels of the workgroup's next tile; 0, 0: none
+};
+
+// Starts a copy of n dwords from global memory to LDS that does not pass through registers
+// (LDS-direct loads: lane l of a wave writes the dword it fetches to M0 + 4*l): dword i of src
+// goes to byte 4*i of the LDS area at lds_addr.  Counts in vmcnt like any load; nothing waits
+// here.  The compiler emits no instruction of its own that uses M0 in these kernels; the
+// s_nop is the wait state the hardware asks for between a write of M0 and an LDS-direct load
+// (the compiler inserts it for its own code, not inside an asm statement).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void copy_to_lds_async(const void *src, const int n,
+        const uint32_t lds_addr, const int tid, const int wave) {
+    for (int base = 0; base < n; base += 256) {
+        const int i = base + tid;
+        const uint32_t m0 = lds_addr + (uint32_t)(base + wave * 64) * 4u; // wave-uniform
+        if (i < n)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                    : : "s"(m0), "v"((uint32_t)i * 4u), "s"(src) : "memory", "m0");
+    }
+}
+#pragma clang diagnostic pop
+
 // KS = 64-channel steps per tap (ceil(IC/64), rounded up to even above 4 and to 12 or 16
 // above 8), PS = 32-pixel
 // blocks per workgroup tile.
@@ -192,7 +224,10 @@ __device__ __forceinline__ uint32_t fp4_of_byte(uint32_t byte) {
 // 32*KS bytes further into the same LDS rows.
 // One tile: the output pixels [p_first, min(p_first + 32*PS, p_limit)) x the 256 filters of
 // filter chunk `chunk`.
-template <int KS, int PS, bool RAW, bool PAIR, bool DEEP>
+// PERSIST: the caller loops over tiles (see conv_mfma_fp4_persistent_kernel); `turn` says what
+// is already in LDS and which tile to prefetch.  The LDS layout then has room for four pixel
+// blocks whatever PS is, so that tiles of two sizes can follow each other.
+template <int KS, int PS, bool RAW, bool PAIR, bool DEEP, bool PERSIST = false>
 __device__ __forceinline__
 void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag,
         const float *__restrict__ alpha, const float *__restrict__ kplane,
@@ -200,23 +235,33 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
         const Geometry &g, const int max_rows, const FastDiv &div_xw,
         const float *__restrict__ a_plane, float *__restrict__ k_out, const float inv_khw,
         const int ic_parts, const uint32_t wfrag_bytes, const uint32_t p_first,
-        const uint32_t p_limit, const int chunk) {
+        const uint32_t p_limit, const int chunk, const TileTurn turn = TileTurn{}) {
+    static_assert(!PERSIST || (!RAW && !DEEP), "persistent tiles: scaled output, one channel part");
     extern __shared__ unsigned char smem[];
     uint32_t *table = reinterpret_cast<uint32_t *>(smem);
     float *alpha_lds = reinterpret_cast<float *>(smem + TABLE_BYTES);
-    unsigned char *rows = smem + TABLE_BYTES + ALPHA_BYTES; // row 0 is zero, then the tile
+    // PERSIST: two staging areas of max_rows * xw packed words, then two of max_rows + 1
+    // floats (mean|x|; the last slot holds zero), ahead of the rows: the LDS-direct loads
+    // that fill them take a 16-bit LDS offset
+    const int stage_words = max_rows * g.xw;
+    const int stage_at = TABLE_BYTES + ALPHA_BYTES;
+    const int stage_bytes = PERSIST ? (2 * stage_words * 4 + 2 * (max_rows + 1) * 4 + 15) & ~15 : 0;
+    unsigned char *rows = smem + stage_at + stage_bytes; // row 0 is zero, then the tile
     // PAIR (an odd number KS of 32-channel words per pixel): two taps share KS steps, so no
     // step is half empty; the rows then hold exactly KS words (16*KS bytes is 4 mod 8 dwords,
     // which keeps the fragment reads conflict-free without padding).
     const int ROW_BYTES = DEEP ? ic_parts * KS * 32 + ROW_PAD
                                : PAIR ? KS * 16 : KS * 32 + ROW_PAD;
-    // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows)
+    // mean|x| of the tile's input pixels, when the K plane is computed here (after the rows;
+    // PERSIST: read from the staging area instead, a_lds is pointed there below)
     float *a_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES);
-    float *k_lds = a_lds + max_rows + 1; // K of the tile's pixels, same case
+    float *k_lds = reinterpret_cast<float *>(rows + (size_t)(1 + max_rows) * ROW_BYTES)
+        + max_rows + 1; // K of the tile's pixels, same case
     // NHWC output: per wave 32 pixel rows of TURN_ROW floats to turn a block around in
     // (an offset from smem, not a rounded pointer: the compiler has to see an LDS address)
-    float *turn_lds = reinterpret_cast<float *>(smem + ((TABLE_BYTES + ALPHA_BYTES
-            + (1 + max_rows) * ROW_BYTES + (max_rows + 1 + 32 * PS) * 4 + 15) & ~15));
+    constexpr int PSL = PERSIST ? 4 : PS; // pixel blocks the layout has room for
+    float *turn_lds = reinterpret_cast<float *>(smem + ((stage_at + stage_bytes
+            + (1 + max_rows) * ROW_BYTES + (max_rows + 1 + 32 * PSL) * 4 + 15) & ~15));
     constexpr int MT = 32 * PS;
     // Weight fragments are fetched in groups of HS steps, one group ahead: a whole tap where
     // the registers allow it (8 VGPRs per step on top of 32 per pixel block), half a tap
@@ -227,7 +272,12 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
         : (KS % 2 == 0 && KS >= 4 && (PS > 3 || 40 * PS + 16 * KS > 216)) ? KS / 2 : KS;
     constexpr int GROUPS_PER_TAP = KS / HS; // 1, 2 or 4
 
-    const int tid = threadIdx.x;
+    int thread = threadIdx.x;
+    // PERSIST: a value the compiler cannot see through, so that nothing computed from it
+    // counts as invariant of the loop over tiles: what is hoisted out of that loop stays in
+    // registers through the main loop, where there are none to spare
+    if constexpr (PERSIST) asm volatile("" : "+v"(thread));
+    const int tid = thread;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // "taps" below are the units the main loop walks over: kernel taps, or pairs of them
@@ -277,14 +327,47 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     // zeros and FP4 has no NaN or infinity, so whatever LDS holds there contributes nothing.
     const int nitems = nrows * g.xw;
     const uint32_t *run = xbits + (size_t)lo * g.xw;
-    constexpr int EARLY = 8;
+    constexpr int EARLY = PERSIST ? 1 : 8;
     uint32_t early[EARLY];
+    // PERSIST: always with mean|x| (a K plane to read would be loads the compiler waits for
+    // with vmcnt(0) in the middle of the staging phase, which would also wait for the copy
+    // of the next tile's words that has just been started)
+    const bool fuse_k = PERSIST || (!RAW && a_plane != nullptr); // uniform
+    float alpha_early = 0.f;
+    const uint32_t *stage = nullptr; // PERSIST: this tile's packed words in LDS
+    if constexpr (PERSIST) {
+        stage = reinterpret_cast<const uint32_t *>(smem + stage_at) + turn.parity * stage_words;
+        float *a_stage = reinterpret_cast<float *>(smem + stage_at + 2 * stage_words * 4);
+        a_lds = a_stage + turn.parity * (max_rows + 1);
+        if (turn.first) { // what stays in LDS for all tiles of this workgroup
+            table[tid] = fp4_of_byte(tid);
+            for (int i = tid; i < ROW_BYTES / 4; i += 256)
+                reinterpret_cast<uint32_t *>(rows)[i] = 0;
+            alpha_lds[tid] = chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
+            if (tid < 2) a_stage[tid * (max_rows + 1) + max_rows] = 0.f;
+            // the words of the first tile: the kernel started their copy before its loop
+            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        }
+        // All waves have finished with the rows, alphas and K of the tile before, and every
+        // wave has waited for its share of this tile's words (ahead of its main loop: the
+        // waits there let no older load pass) before it arrives here.
+        __syncthreads();
+        if (turn.next_end != 0) { // the next tile's words go to the other area meanwhile
+            int nlo, nhi;
+            tile_span(g, turn.next_first, turn.next_end, nlo, nhi);
+            const int nn = min(nhi - nlo + 1, max_rows);
+            const uint32_t other = turn.parity ^ 1u;
+            copy_to_lds_async(xbits + (size_t)nlo * g.xw, nn * g.xw,
+                    (uint32_t)(size_t)smem + stage_at + other * stage_words * 4, tid, wave);
+            copy_to_lds_async(a_plane + nlo, nn, (uint32_t)(size_t)smem + stage_at
+                        + 2 * stage_words * 4 + other * (max_rows + 1) * 4, tid, wave);
+        }
+    } else {
 #pragma unroll
     for (int u = 0; u < EARLY; u++) {
         const int i = u * 256 + tid;
         early[u] = i < nitems ? run[i] : 0u;
     }
-    const bool fuse_k = !RAW && a_plane != nullptr; // uniform
     float a_early = 0.f;
     if (fuse_k && tid < nrows) a_early = a_plane[lo + tid];
     table[tid] = fp4_of_byte(tid);
@@ -292,13 +375,14 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     // asked for now, put into LDS after the expansion: nothing needs it before the epilogue,
     // and the first barrier does not have to wait for it
     // (the raw-accumulator variant takes a table that need not hold alpha at all)
-    const float alpha_early = !RAW && chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
+    alpha_early = !RAW && chunk * NT + tid < g.oc ? alpha[chunk * NT + tid] : 0.f;
     if (fuse_k) { // mean|x| of the staged input pixels, plus one slot that holds zero
         if (tid < nrows) a_lds[tid] = a_early;
         if (tid == 0) a_lds[max_rows] = 0.f;
         for (int i = 256 + tid; i < nrows; i += 256) a_lds[i] = a_plane[lo + i];
     }
     __syncthreads();
+    }
     auto expand = [&](int i, uint32_t word) { // item i of the run -> 32 FP4 codes of its row
         const int r = (int)div_xw.div((uint32_t)i), j = i - r * g.xw; // row, 32-channel word
         v4i q;
@@ -308,10 +392,12 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
         q.w = table[word & 0xFF];
         *reinterpret_cast<v4i *>(rows + (size_t)(1 + r) * ROW_BYTES + j * 16) = q;
     };
+    if constexpr (!PERSIST) {
 #pragma unroll
-    for (int u = 0; u < EARLY; u++) {
-        const int i = u * 256 + tid;
-        if (i < nitems) expand(i, early[u]);
+        for (int u = 0; u < EARLY; u++) {
+            const int i = u * 256 + tid;
+            if (i < nitems) expand(i, early[u]);
+        }
     }
     // K of the tile's pixels, when it is not read from the K plane: wave ps sums the block
     // of 32 pixels ps exactly as the box filter does (in-bounds taps in row-major order, each
@@ -347,12 +433,13 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
             }
         }
     }
-    for (int base = EARLY * 256; base < nitems; base += 4 * 256) {
+    for (int base = PERSIST ? 0 : EARLY * 256; base < nitems; base += 4 * 256) {
         uint32_t w[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int i = base + u * 256 + tid;
-            w[u] = i < nitems ? run[i] : 0u;
+            if constexpr (PERSIST) w[u] = i < nitems ? stage[i] : 0u;
+            else w[u] = i < nitems ? run[i] : 0u;
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -361,7 +448,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
         }
     }
 
-    alpha_lds[tid] = alpha_early;
+    if constexpr (!PERSIST) alpha_lds[tid] = alpha_early;
 
     // ---- this wave: 64 filters x 32*PS pixels --------------------------------------------------
     const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
@@ -522,14 +609,25 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     };
 
     v4i wa[HS][2], wb[HS][2];
-    if (wave_has_filters) {
-        static_for<HS>([&](auto step) { request_step(0, step, wa); });
-        if constexpr (PAIR) {
-            pair_rows(pairaddr);
-        } else {
-            tap_rows(0, 0, rowaddr);
-            advance_tap();
-        }
+    // A wave without filters (fewer than 256 of them in this chunk) leaves here, through a
+    // barrier of its own: the barrier counts arrivals, whichever instruction they come from.
+    // One test of the condition, ahead of the first hand-issued load, so that no path (of the
+    // hardware, or of the walk in tests/test_isa_hazards.py, which knows nothing of branch
+    // conditions) mixes "has asked for fragments" with "skips the waits of the main loop".
+    if (!wave_has_filters) {
+        __syncthreads();
+        // PERSIST: this wave's share of the next tile's words has to be in LDS before it
+        // meets the others at the next tile's first barrier (the others wait for theirs
+        // ahead of their main loops: the waits there let no older load pass)
+        if constexpr (PERSIST) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        return;
+    }
+    static_for<HS>([&](auto step) { request_step(0, step, wa); });
+    if constexpr (PAIR) {
+        pair_rows(pairaddr);
+    } else {
+        tap_rows(0, 0, rowaddr);
+        advance_tap();
     }
     __syncthreads(); // FP4 rows are in place
     float kv[PS]; // K of this wave's pixels
@@ -544,7 +642,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
             for (int ps = 0; ps < PS; ps++) kv[ps] = kplane[live[ps] ? pix[ps] : 0];
         }
     }
-    if (wave_has_filters) {
+    {
         if constexpr (PAIR) {
             uint32_t a0[PS];
             pair_addr(0, pairaddr, a0);
@@ -610,7 +708,6 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     //      computed once, the filter is a scalar offset, and a dead pixel or a filter past
     //      OC gets an offset beyond the buffer, which the hardware drops; no 64-bit address
     //      arithmetic and no branches per store. ------------------------------------------------
-    if (!wave_has_filters) return;
     const int lane_hi = lane >> 5;
     constexpr uint32_t DROP = 0xFFFFFFF0u; // >= the buffer size: the store is discarded
     const __amdgpu_buffer_rsrc_t outbuf = __builtin_amdgcn_make_buffer_rsrc(
@@ -807,6 +904,95 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
     }
 }
 
+// The same tiles for launches with several rounds of them: two workgroups per compute unit
+// that stay, each walking over its tiles.  Tiles are numbered per XCD as in the two-size
+// kernel above (the first big_per_xcd have PS blocks, the rest PSB); workgroup n of an XCD
+// has filter chunk n % oc_chunks and takes the tiles n / oc_chunks + j * tiles_per_round,
+// j = 0, 1, ...: a round of tiles is a contiguous stretch of pixels, so neighbouring tiles
+// are worked on at the same time and meet in one L2, and the host picks big_per_xcd as a
+// whole number of rounds so that every workgroup gets the same sequence of sizes.
+// What a workgroup gains over a fresh one per tile: the table, the zero row, the alphas and
+// the kernel arguments are set up once; the packed words of the next tile (and mean|x| of its
+// input pixels) are copied into LDS while the current tile is multiplied, so staging waits
+// for no global load; and no dispatch has to be waited for between tiles.
+template <int KS, int PS, int PSB, bool PAIR>
+__global__ __launch_bounds__(256, 2)
+void conv_mfma_fp4_persistent_kernel(const uint32_t *__restrict__ xbits,
+        const v4i *__restrict__ wfrag, const float *__restrict__ alpha,
+        const float *__restrict__ kplane, float *__restrict__ dst, const Geometry g,
+        const int max_rows, const int oc_chunks, const uint32_t tiles_per_round,
+        const FastDiv div_xw, const float *__restrict__ a_plane, float *__restrict__ k_out,
+        const float inv_khw, const uint32_t wfrag_bytes, const uint32_t big_per_xcd,
+        const uint32_t blocks_per_xcd, const uint32_t rounds, const int reverse_second,
+        const uint32_t stagger) {
+    extern __shared__ unsigned char smem[];
+    const uint32_t xcd = blockIdx.x & 7, nth = blockIdx.x >> 3;
+    const uint32_t first = xcd * blocks_per_xcd; // pixel blocks of this XCD: [first, last)
+    const uint32_t p_limit = min((first + blocks_per_xcd) * 32u, g.npix_out);
+    uint32_t tile = oc_chunks == 1 ? nth : nth / oc_chunks;
+    const int chunk = nth - tile * oc_chunks;
+    if (tile >= tiles_per_round) return; // more workgroups than a round has (tile, chunk) pairs
+    // first pixel of tile t of this XCD; tiles past the XCD's pixels start at or after p_limit
+    auto first_pixel = [&](uint32_t t) {
+        return t < big_per_xcd ? (first + t * PS) * 32u
+                               : (first + big_per_xcd * PS + (t - big_per_xcd) * PSB) * 32u;
+    };
+    auto end_pixel = [&](uint32_t t, uint32_t p) {
+        return min(p + (t < big_per_xcd ? 32u * PS : 32u * PSB), p_limit);
+    };
+    if (first_pixel(tile) >= p_limit) return;
+    // The two workgroups of a compute unit should not run the same phase at the same time: a
+    // wave that has issued a tile's stores cannot take in the next tile's weight fragments
+    // before those stores are acknowledged (one in-order counter for loads and stores), and
+    // the matrix pipes should have the other workgroup's main loop to run meanwhile.  The
+    // hardware places workgroups n and n + (workgroups per XCD) / 2 of an XCD on one CU; the
+    // second of them walks its tiles in the opposite order (small tiles first) and may start
+    // late.
+    uint32_t step = tiles_per_round; // (to the next tile; the unsigned sum wraps when reversed)
+    if (reverse_second != 0 && nth >= (tiles_per_round * oc_chunks) / 2) {
+        uint32_t last = tile + (rounds - 1) * tiles_per_round;
+        while (last != tile && first_pixel(last) >= p_limit) last -= tiles_per_round;
+        tile = last;
+        step = 0u - tiles_per_round;
+    }
+    if (nth >= (tiles_per_round * oc_chunks) / 2)
+        for (uint32_t i = 0; i < stagger; i++) __builtin_amdgcn_s_sleep(16);
+    uint32_t p_first = first_pixel(tile);
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    { // the first tile's words: into staging area 0 (the layout is conv_tile's)
+        int lo, hi;
+        tile_span(g, p_first, end_pixel(tile, p_first), lo, hi);
+        const int nrows = min(hi - lo + 1, max_rows);
+        const uint32_t stage = (uint32_t)(size_t)smem + TABLE_BYTES + ALPHA_BYTES;
+        copy_to_lds_async(xbits + (size_t)lo * g.xw, nrows * g.xw, stage, tid, wave);
+        copy_to_lds_async(a_plane + lo, nrows, stage + 2u * (uint32_t)(max_rows * g.xw) * 4u,
+                tid, wave);
+    }
+    TileTurn turn{true, 0u, 0u, 0u};
+    for (;;) {
+        const uint32_t next = tile + step;
+        // (walking backwards, tile numbers below the first wrap around to huge values)
+        const uint32_t next_first = next < rounds * tiles_per_round ? first_pixel(next) : p_limit;
+        const bool more = next_first < p_limit;
+        turn.next_first = more ? next_first : 0u;
+        turn.next_end = more ? end_pixel(next, next_first) : 0u;
+        if (tile < big_per_xcd)
+            conv_tile<KS, PS, false, PAIR, false, true>(xbits, wfrag, alpha, kplane, dst, nullptr,
+                    g, max_rows, div_xw, a_plane, k_out, inv_khw, 1, wfrag_bytes, p_first,
+                    p_limit, chunk, turn);
+        else
+            conv_tile<KS, PSB, false, PAIR, false, true>(xbits, wfrag, alpha, kplane, dst,
+                    nullptr, g, max_rows, div_xw, a_plane, k_out, inv_khw, 1, wfrag_bytes,
+                    p_first, p_limit, chunk, turn);
+        if (!more) break;
+        tile = next;
+        p_first = next_first;
+        turn.first = false;
+        turn.parity ^= 1u;
+    }
+}
+
 // Calibration only: the matrix instruction of the convolution kernel and nothing else.  Every
 // wave multiplies pseudo-random +-1 fragments (the FP4 codes 0x2 and 0xA) that never leave
 // its registers into eight independent accumulator blocks, `iterations` times.  What this
@@ -960,10 +1146,12 @@ int max_tile_rows(const Geometry &g, uint32_t mt, uint32_t step = 0) {
     return most;
 }
 
-size_t lds_bytes_for(const Geometry &g, size_t rows, int ps) {
+size_t lds_bytes_for(const Geometry &g, size_t rows, int ps, bool persist = false) {
     const size_t row_bytes = pair_taps(g) ? g.xw * 16
         : channel_parts(g) * steps_per_tap(g) * 32 + ROW_PAD;
-    size_t bytes = TABLE_BYTES + ALPHA_BYTES + (1 + rows) * row_bytes
+    // persistent workgroups: two staging areas for packed words and for mean|x| (conv_tile)
+    const size_t stage = persist ? (2 * rows * g.xw * 4 + 2 * (rows + 1) * 4 + 15) & ~(size_t)15 : 0;
+    size_t bytes = TABLE_BYTES + ALPHA_BYTES + stage + (1 + rows) * row_bytes
         + (rows + 1 + 32 * ps) * sizeof(float);
     if (g.dst_fmt == xnor_nn_data_format_nhwc && (g.oc & 3) == 0) // turn-around rows, 4 waves
         bytes = ((bytes + 15) & ~(size_t)15) + 4 * 32 * TURN_ROW * sizeof(float);
@@ -1078,6 +1266,34 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
     return hipGetLastError();
 }
 
+template <int KS, bool PAIR>
+hipError_t launch_mfma_persistent(const Geometry &g, const uint32_t *xbits,
+        const uint32_t *wfrag, const float *alpha, const float *k, float *dst,
+        const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
+    const int chunks = (g.oc + NT - 1) / NT;
+    const dim3 grid(g.mfma_tiles_per_round * chunks * 8), block(256);
+    const size_t lds = g.mfma_lds;
+    const auto kernel = conv_mfma_fp4_persistent_kernel<KS, 4, 3, PAIR>;
+    if (lds > (size_t)LDS_DEFAULT) { // asked for once per device and size
+        static std::atomic<size_t> granted[MAX_DEVICES];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+            return hipErrorInvalidDevice;
+        if (lds > granted[dev].load(std::memory_order_acquire)) {
+            const hipError_t e = hipFuncSetAttribute((const void *)kernel,
+                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+            granted[dev].store(lds, std::memory_order_release);
+        }
+    }
+    launch_kernel(kernel, grid, block, lds, s, ev, xbits, reinterpret_cast<const v4i *>(wfrag),
+            alpha, k, dst, g, g.mfma_rows, chunks, g.mfma_tiles_per_round,
+            FastDiv::make((uint32_t)g.xw), a_or_null, k_out, 1.f / g.kh / g.kw, g.mfma_wbytes,
+            g.mfma_big_per_xcd, g.mfma_blocks_per_xcd, g.mfma_rounds, g.mfma_reverse,
+            g.mfma_stagger);
+    return hipGetLastError();
+}
+
 template <int KS>
 hipError_t launch_mfma_deep(const Geometry &g, const uint32_t *xbits, const uint32_t *wfrag,
         const float *alpha, const float *k, float *dst, int32_t *popc,
@@ -1096,6 +1312,11 @@ hipError_t launch_mfma_ps(const Geometry &g, const uint32_t *xbits, const uint32
         const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     if (g.mfma_ps_small > 0) { // two tile sizes: four blocks, and two or three
         if constexpr (KS < 16 && !(PAIR && KS >= 5)) {
+            // persistent workgroups; the raw accumulators, and a pass that reads a K plane
+            // instead of mean|x|, go through the same tiles with a workgroup per tile
+            if (g.mfma_persist && popc == nullptr && a_or_null != nullptr)
+                return launch_mfma_persistent<KS, PAIR>(g, xbits, wfrag, alpha, k, dst,
+                        a_or_null, k_out, s, ev);
             if (g.mfma_ps_small == 3)
                 return launch_mfma<KS, 4, PAIR, false, 3>(g, xbits, wfrag, alpha, k, dst, popc,
                         a_or_null, k_out, s, ev);
@@ -1146,6 +1367,8 @@ void mfma_plan(Geometry &g) {
     g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
     g.mfma_ps_small = 0;
     g.mfma_big_per_xcd = g.mfma_blocks_per_xcd = 0;
+    g.mfma_persist = g.mfma_reverse = 0;
+    g.mfma_tiles_per_round = g.mfma_rounds = g.mfma_stagger = 0;
     g.stream_dst = 0;
     g.mfma_parts = 1;
     g.mfma_lds = g.mfma_wbytes = 0;
@@ -1190,6 +1413,56 @@ void mfma_plan(Geometry &g) {
     if (getenv("XNOR_NN_HIP_MFMA_PS") || g.mfma_parts > 1 || g.mfma_steps >= 16
             || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4))
         mix = fill = false;
+    // Persistent workgroups (see the kernel): only on request, XNOR_NN_HIP_MFMA_PERSIST=N with
+    // N workgroups per XCD (64 = two per compute unit).  Measured on MI355X they are slower than
+    // a workgroup per tile wherever a launch has several rounds of tiles (ResNet 3x3 MB 64:
+    // 68.4 against 66.0 us, conv2 shape MB 128: 41.4 against 40.7 us): the two workgroups of a
+    // compute unit then run every phase at the same time, so staging (4.9 us per tile) and
+    // stores (2.5 to 4.3 us) overlap no matrix instructions, where workgroups dispatched one
+    // by one drift apart.  Kept because tests walk small problems in many rounds this way.
+    // With `per_round` (tile, chunk) slots per XCD a workgroup gets n = ceil(blocks /
+    // per_round) pixel blocks, walked as a rounds of four-block tiles and b rounds of
+    // three-block tiles, 4a + 3b >= n as small as possible, a as large as possible.
+    {
+        uint32_t wgs_per_xcd = 0;
+        if (const char *e = getenv("XNOR_NN_HIP_MFMA_PERSIST"))
+            wgs_per_xcd = (uint32_t)(atoi(e) > 0 ? atoi(e) : 0);
+        const uint32_t per_round = wgs_per_xcd / chunks;
+        const uint32_t n = per_round ? (blocks_per_xcd + per_round - 1) / per_round : 0;
+        bool persist = n >= 1;
+        if (getenv("XNOR_NN_HIP_MFMA_PS") || getenv("XNOR_NN_HIP_MFMA_MIX") || g.mfma_parts > 1
+                || g.mfma_steps >= 16 || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4))
+            persist = false;
+        if (persist) {
+            const int rows = max_tile_rows(g, 32 * 4, 32);
+            const size_t lds = lds_bytes_for(g, (size_t)rows, 4, true);
+            if (lds <= (size_t)LDS_TWO_PER_CU) {
+                uint32_t best_a = 0, best_total = 0;
+                for (uint32_t a = 0; 4 * a <= n + 3; a++) {
+                    const uint32_t rest = n > 4 * a ? n - 4 * a : 0, b = (rest + 2) / 3;
+                    const uint32_t total = 4 * a + 3 * b;
+                    if (best_total == 0 || total < best_total || (total == best_total && a > best_a)) {
+                        best_a = a;
+                        best_total = total;
+                    }
+                }
+                g.mfma_persist = 1;
+                g.mfma_tiles_per_round = per_round;
+                g.mfma_rounds = best_a + (best_total - 4 * best_a) / 3;
+                g.mfma_reverse = 0;
+                g.mfma_stagger = 0;
+                if (const char *e = getenv("XNOR_NN_HIP_MFMA_REVERSE")) g.mfma_reverse = e[0] == '1';
+                if (const char *e = getenv("XNOR_NN_HIP_MFMA_STAGGER")) g.mfma_stagger = (uint32_t)atoi(e);
+                g.mfma_ps = 4;
+                g.mfma_ps_small = 3;
+                g.mfma_big_per_xcd = best_a * per_round;
+                g.mfma_blocks_per_xcd = blocks_per_xcd;
+                g.mfma_rows = rows;
+                g.mfma_lds = (uint32_t)lds;
+                return;
+            }
+        }
+    }
     if (mix || fill) {
         const int rows = max_tile_rows(g, 32 * 4, 32);
         const size_t lds = lds_bytes_for(g, (size_t)rows, 4);
@@ -1229,6 +1502,9 @@ const char *mfma_kernel_name(const Geometry &g) {
     if (g.mfma_parts > 1)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d,PARTS=%d>",
                 g.mfma_steps, g.mfma_ps, g.mfma_parts);
+    else if (g.mfma_persist)
+        snprintf(name, sizeof name, "conv_mfma_fp4_persistent_kernel<KS=%d,PS=%d+%d%s>",
+                g.mfma_steps, g.mfma_ps, g.mfma_ps_small, g.mfma_pair ? ",PAIR" : "");
     else if (g.mfma_ps_small > 0)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d+%d%s>", g.mfma_steps,
                 g.mfma_ps, g.mfma_ps_small, g.mfma_pair ? ",PAIR" : "");

@@ -67,6 +67,11 @@ struct Geometry {
                                 // XCD take this many blocks (see the kernel)
     uint32_t mfma_big_per_xcd;  // ... after this many workgroups with mfma_ps blocks,
     uint32_t mfma_blocks_per_xcd; // out of this many pixel blocks per XCD
+    int mfma_persist;           // 1: two workgroups per CU stay and walk over the tiles, taking
+    uint32_t mfma_tiles_per_round; // every mfma_tiles_per_round-th tile of their XCD
+    uint32_t mfma_rounds;       // rounds of tiles a persistent workgroup walks at most
+    int mfma_reverse;           // 1: the second workgroup of a CU walks its tiles last to first
+    uint32_t mfma_stagger;      // ... and starts this many sleep periods late
     size_t wfrag_offset;        // byte offset of the FP4 weight fragments in bin_weights
     // the matrix-core kernel's variant and sizes, fixed once by mfma_plan: steps per tap (or
     // per pair of taps), tap pairing, channel parts, input pixels a tile stages at most, LDS
