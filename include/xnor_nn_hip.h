@@ -40,9 +40,18 @@ xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *st
  * descriptor withdraws it.  A caller that changes the contents of user_src between
  * binarize_data and calculate_k, or that reads res[k] as a raw device pointer between
  * calculate_k and forward, switches fusion off (on = 0; the environment variable
- * XNOR_NN_HIP_SEPARATE_K=1 does the same for every descriptor): every executor then
- * completes its own stage as in the reference.  xnor_nn_hip_export_floats always returns
- * the finished K plane. */
+ * XNOR_NN_HIP_SEPARATE_K=1, read when a descriptor is initialised, does the same for every
+ * descriptor initialised while it is set): every executor then completes its own stage as
+ * in the reference.  xnor_nn_hip_export_floats always returns the finished K plane.
+ * The records are keyed on the addresses in slots `a` and `k`.  While fusion is on, buffers
+ * that have been in those slots must therefore be released through xnor_nn_free_resources
+ * (or after xnor_nn_destroy_convolution of every descriptor that used them): a caller that
+ * brings its own `a`/`k` buffers and frees them behind the library's back leaves a record
+ * that a later call on a recycled address would act on.
+ * A box filter that is owed runs on the stream its mean|x| was written on, with the geometry
+ * of the descriptor that owes it; when another descriptor's call triggers it (its table
+ * names that K plane, or is about to overwrite that mean|x| plane) and that descriptor runs
+ * on another stream, the two streams are ordered with events around the filter. */
 xnor_nn_status_t xnor_nn_hip_set_stage_fusion(const xnor_nn_convolution_t *c, int on);
 
 /* Block until everything enqueued by this descriptor's executors has finished. */
@@ -138,8 +147,9 @@ xnor_nn_status_t xnor_nn_hip_mfma_only(int workgroups, int iterations, void *str
  * run on until the process ends (its device address is looked up once per GPU, by
  * xnor_nn_init_convolution or by the first call here, whichever comes first).  Every call on a GPU shares that array: calls that overlap
  * on one GPU (two streams, two threads) race on it and must be ordered by the caller.
- * More than XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS weights, or a host pointer that is null, is
- * refused with xnor_nn_error_invalid_input and a line on stderr. */
+ * More than XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS weights, a null pointer, or a pointer to host
+ * memory (the kernels would fault on it) is refused with xnor_nn_error_invalid_input and a
+ * line on stderr; nothing is launched then. */
 #define XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS 2147483647LL /* the reference counts them in an int */
 xnor_nn_status_t xnor_nn_hip_binarize_weights_float_noalloc(const xnor_nn_convolution_t *c,
         const float *from, float *to);

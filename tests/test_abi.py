@@ -243,7 +243,8 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     runtime-shape kernel): which kernel variant each of the five benchmark workloads and the
     boundary shapes get, decided at init from the shape alone."""
     for key in ("XNOR_NN_HIP_CONV", "XNOR_NN_HIP_MFMA_PS", "XNOR_NN_HIP_MFMA_MIX",
-                "XNOR_NN_HIP_MFMA_PAIR", "XNOR_NN_HIP_NHWC", "XNOR_NN_HIP_STREAM_DST"):
+                "XNOR_NN_HIP_MFMA_PAIR", "XNOR_NN_HIP_NHWC", "XNOR_NN_HIP_STREAM_DST",
+                "XNOR_NN_HIP_MFMA_PERSIST"):
         monkeypatch.delenv(key, raising=False)
     conv4 = (256, 384, 13, 13, 3, 3, 1, 1, 1, 1)
     assert kernel_names((1,) + conv4) == ("binarize_nchw_kernel", "conv_mfma_fp4_kernel<KS=6,PS=1>")
@@ -273,3 +274,32 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     # the switch that forces the XNOR/popcount kernel (used to profile the two side by side)
     monkeypatch.setenv("XNOR_NN_HIP_CONV", "valu")
     assert kernel_names((256,) + conv4)[1] == "conv_xnor_popc_kernel<XW=12,Q=16>"
+
+
+def test_inputs_that_reach_the_dropped_offset_take_the_generic_kernel():
+    """The tiled binarize kernels read a channel past the end of a ragged slice through the
+    byte offset 0xFFFFFFF0, which the hardware drops only while it lies outside the buffer.
+    An input that ends at or beyond that offset (but below 4 GiB) must not run them."""
+    # 1 x 3 x 21 x 17043521 floats = 0xFFFFFFFC bytes: inside the gap
+    assert kernel_names((1, 4, 3, 21, 17043521, 1, 1, 1, 1, 0, 0))[0] == "binarize_generic_kernel"
+    nhwc = (capi.FMT_NHWC, capi.FMT_OIHW, capi.FMT_NCHW)
+    # 1 x 4 x 1 x 268435455 floats = 0xFFFFFFF0 bytes, channels a multiple of four
+    assert kernel_names((1, 4, 4, 1, 268435455, 1, 1, 1, 1, 0, 0), nhwc)[0] \
+        == "binarize_generic_kernel"
+    # just below: 0xFFFFFFEC bytes
+    assert kernel_names((1, 4, 1, 1, 1073741819, 1, 1, 1, 1, 0, 0))[0] == "binarize_nchw_kernel"
+    assert kernel_names((1, 4, 4, 1, 268435454, 1, 1, 1, 1, 0, 0), nhwc)[0] \
+        == "binarize_nhwc_tiled_kernel"
+
+
+def test_persistent_workgroups_are_planned_on_request_only(monkeypatch):
+    """XNOR_NN_HIP_MFMA_PERSIST=N: N workgroups per XCD that walk over the tiles; without it a
+    workgroup per tile, whatever the size (measured faster)."""
+    resnet = (64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1)
+    monkeypatch.delenv("XNOR_NN_HIP_MFMA_PERSIST", raising=False)
+    assert kernel_names(resnet)[1] == "conv_mfma_fp4_kernel<KS=4,PS=4>"
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_PERSIST", "64")
+    assert kernel_names(resnet)[1] == "conv_mfma_fp4_persistent_kernel<KS=4,PS=4+3>"
+    # sixteen steps per tap have no four-block tile: never persistent
+    assert kernel_names((8, 256, 1024, 14, 14, 3, 3, 1, 1, 1, 1))[1].startswith(
+        "conv_mfma_fp4_kernel<KS=16")

@@ -141,6 +141,57 @@ def test_two_resource_tables_on_one_descriptor(oracle, gpu):
     conv.close()
 
 
+def test_two_descriptors_on_two_streams_share_a_mean_plane(oracle, gpu):
+    """Descriptor A (stream sa) leaves its box filter owed to its K plane; descriptor B
+    (stream sb, a table that names A's mean|x| plane as its own) then binarizes other data
+    and so overwrites that plane.  The filter owed by A has to run first, where A's mean|x|
+    was written (on sa, behind A's binarize kernel), and B's kernel has to wait for it: the
+    two streams are ordered with events.  A large batch keeps A's binarize kernel busy when
+    B is called.  Then the other way round: B's K owed, read back through A."""
+    import torch
+    d, x1, w = synth.make_workload("alexnet_conv4_mb256", 96)
+    x2 = (x1[::-1] * np.float32(0.75)).copy()
+    s = oracle_shape(oracle, d)
+    want1, want2 = oracle.forward(s, x1, w), oracle.forward(s, x2, w)
+    wt = torch.from_numpy(w).to(gpu)
+    x1t, x2t = torch.from_numpy(x1).to(gpu), torch.from_numpy(x2).to(gpu)
+    ya = torch.empty(want1["dst"].shape, dtype=torch.float32, device=gpu)
+    yb = torch.empty_like(ya)
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    A, B = make(d, wt), make(d, wt)
+    A.set_stream(sa)
+    B.set_stream(sb)
+    own_a = B.res[capi.RES_A]
+    B.res[capi.RES_A] = A.res[capi.RES_A]  # one mean|x| plane for both tables
+    torch.cuda.synchronize()
+    for rep in range(3):
+        run(A, A.res, "binarize_data", x1t, ya)
+        run(A, A.res, "calculate_k")          # K(x1) owed to A's K plane, mean|x| written on sa
+        run(B, B.res, "binarize_data", x2t, yb)  # overwrites the plane: A's filter runs first
+        run(B, B.res, "calculate_k")
+        run(B, B.res, "forward")
+        run(A, A.res, "forward")              # bits(x1), K(x1) from the finished K plane
+        torch.cuda.synchronize()
+        assert same_bits(A.export_floats(capi.RES_K), want1["k"]), rep
+        assert same_bits(ya.cpu().numpy(), want1["dst"]), rep
+        assert same_bits(yb.cpu().numpy(), want2["dst"]), rep
+        # B's K owed (on sb); A asks for a forward with B's K plane in its table
+        run(B, B.res, "binarize_data", x2t, yb)
+        run(B, B.res, "calculate_k")
+        mixed = capi.Resources()
+        for i in range(capi.RES_NUMBER):
+            mixed[i] = A.res[i]
+        mixed[capi.RES_K] = B.res[capi.RES_K]
+        run(A, mixed, "forward", dst=ya)      # bits(x1) of A's table, K(x2) owed by B
+        torch.cuda.synchronize()
+        n_alpha = (2 * want1["popc"].astype(np.int64) - want1["opc"][None, None]).astype(
+            np.float32) * want1["alpha"][None, :, None, None]
+        assert same_bits(ya.cpu().numpy(), (n_alpha * want2["k"][:, None]).astype(np.float32)), rep
+    B.res[capi.RES_A] = own_a
+    A.close()
+    B.close()
+
+
 def test_free_and_allocate_between_calculate_k_and_forward(oracle, gpu):
     """calculate_k leaves its box filter to forward; when the table is freed in between,
     nothing may run later on the freed buffers, and a fresh table on the same descriptor

@@ -621,15 +621,24 @@ def test_deferred_box_filter_keeps_stage_semantics(oracle, gpu, monkeypatch):
     conv.synchronize()
     assert np.array_equal(dt.cpu().numpy().view(np.uint32), want2["dst"].view(np.uint32))
     assert np.array_equal(conv.export_floats(capi.RES_K), want2["k"])
-    # (4)
+    conv.close()
+    # (4) the switch is read when a descriptor is initialised: the K plane is then complete,
+    # in device memory, when calculate_k returns (read raw here, not through the export
+    # helper, which would settle a deferred filter)
     monkeypatch.setenv("XNOR_NN_HIP_SEPARATE_K", "1")
+    conv = make(d, torch.from_numpy(w).to(gpu))
     dt.zero_()
-    conv.stage("binarize_data", src=x1t)
+    kt = torch.zeros(want1["k"].shape, dtype=torch.float32, device=gpu)  # a K plane of ours
+    own_k = conv.res[capi.RES_K]
+    conv.res[capi.RES_K] = kt.data_ptr()
+    conv.stage("binarize_data", src=x1t, dst=dt)
     conv.stage("calculate_k")
+    conv.synchronize()
+    assert np.array_equal(kt.cpu().numpy(), want1["k"])
     conv.stage("forward")
     conv.synchronize()
     assert np.array_equal(dt.cpu().numpy().view(np.uint32), want1["dst"].view(np.uint32))
-    assert np.array_equal(conv.export_floats(capi.RES_K), want1["k"])
+    conv.res[capi.RES_K] = own_k
     conv.close()
 
 

@@ -72,15 +72,16 @@ xnor_nn_status_t unimplemented_stage(const xnor_nn_convolution_t *, xnor_nn_reso
 //          plane.  Whatever else needs the K plane, or is about to overwrite that mean|x|,
 //          runs the box filter first.
 // Entries die with the buffers (xnor_nn_free_resources) and with the descriptor.
+// An Owed entry also names the stream on which its mean|x| was written: the box filter that
+// settles it runs there, whichever descriptor's call triggers it.
 struct Ready { const State *st; const void *src; };
-struct Owed { const State *st; const float *a; };
+struct Owed { const State *st; const float *a; hipStream_t stream; };
 std::mutex handover_mu;
 std::unordered_map<const void *, Ready> ready_by_a;
 std::unordered_map<const void *, Owed> owed_by_k;
 
-bool fusion_on(const State *st) {
-    return st->fuse_stages && getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr;
-}
+// (XNOR_NN_HIP_SEPARATE_K is read once, when the descriptor is initialised)
+bool fusion_on(const State *st) { return st->fuse_stages; }
 
 void withdraw_ready(const void *a) {
     if (a == nullptr) return;
@@ -98,14 +99,37 @@ bool take_owed(const void *k, Owed *out) {
     return true;
 }
 
-xnor_nn_status_t run_box_filter(const State *st, const Owed &o, float *k) {
+// The box filter owed to k, with the geometry of the descriptor that owes it (fixed at its
+// initialisation) and on the stream its mean|x| was written on.  When that is not the
+// calling descriptor's stream, the two are ordered with events in both directions: the
+// filter runs after what the caller has enqueued so far (which may still read the old K
+// plane), and what the caller enqueues next (a kernel that reads K, or one that overwrites
+// mean|x|) runs after the filter.  Called with st->mu held.
+xnor_nn_status_t run_box_filter(State *st, const Owed &o, float *k) {
     if (st->verbose) printf("xnor_nn exec (deferred calculate_k): box_filter_kernel\n");
-    return launch_box_filter(o.st->g, o.a, k, st->stream) == hipSuccess ? xnor_nn_success
-                                                                        : xnor_nn_error_memory;
+    const bool other_stream = o.stream != st->stream;
+    if (other_stream) {
+        if (!st->order_before
+                && (hipEventCreateWithFlags(&st->order_before, hipEventDisableTiming) != hipSuccess
+                    || hipEventCreateWithFlags(&st->order_after, hipEventDisableTiming)
+                        != hipSuccess)) {
+            (void)hipGetLastError();
+            return xnor_nn_error_memory;
+        }
+        if (hipEventRecord(st->order_before, st->stream) != hipSuccess
+                || hipStreamWaitEvent(o.stream, st->order_before, 0) != hipSuccess)
+            return xnor_nn_error_memory;
+    }
+    if (launch_box_filter(o.st->g, o.a, k, o.stream) != hipSuccess) return xnor_nn_error_memory;
+    if (other_stream
+            && (hipEventRecord(st->order_after, o.stream) != hipSuccess
+                || hipStreamWaitEvent(st->stream, st->order_after, 0) != hipSuccess))
+        return xnor_nn_error_memory;
+    return xnor_nn_success;
 }
 
 // Runs the box filter owed to the K plane k, if any.
-xnor_nn_status_t settle_k(const State *st, float *k) {
+xnor_nn_status_t settle_k(State *st, float *k) {
     Owed o;
     if (!take_owed(k, &o)) return xnor_nn_success;
     return run_box_filter(st, o, k);
@@ -113,7 +137,7 @@ xnor_nn_status_t settle_k(const State *st, float *k) {
 
 // Runs every box filter that still has to read the mean|x| plane a (about to be overwritten),
 // except the one owed to skip_k, which is dropped: its K plane is about to be recomputed.
-xnor_nn_status_t settle_readers_of(const State *st, const float *a, const void *skip_k) {
+xnor_nn_status_t settle_readers_of(State *st, const float *a, const void *skip_k) {
     std::vector<std::pair<float *, Owed>> todo;
     {
         std::lock_guard<std::mutex> lock(handover_mu);
@@ -229,7 +253,7 @@ xnor_nn_status_t exec_calculate_k(const xnor_nn_convolution_t *c, xnor_nn_resour
             printf("xnor_nn exec calculate_k: %sbox filter deferred to the convolution\n",
                     a_ready ? "" : "mean_abs, ");
         std::lock_guard<std::mutex> lock(handover_mu);
-        owed_by_k[k] = Owed{st, a};
+        owed_by_k[k] = Owed{st, a, st->stream};
         return xnor_nn_success;
     }
     {
@@ -300,7 +324,7 @@ xnor_nn_status_t run_convolution(const xnor_nn_convolution_t *c, xnor_nn_resourc
     const float *a = nullptr;
     Owed o;
     if (!raw && take_owed(k, &o)) {
-        if (st->g.use_mfma && o.st == st) {
+        if (st->g.use_mfma && o.st == st && o.stream == st->stream) {
             a = o.a;
         } else {
             const xnor_nn_status_t rc = run_box_filter(st, o, k);
@@ -448,6 +472,7 @@ xnor_nn_status_t xnor_nn_init_convolution(xnor_nn_convolution_t *c,
     g.div_ow = FastDiv::make(g.ow);
     const char *v = getenv("XNOR_NN_VERBOSE");
     st->verbose = v && v[0] == '1';
+    st->fuse_stages = getenv("XNOR_NN_HIP_SEPARATE_K") == nullptr; // read here, once
 
     // Byte sizes of the device buffers (the reference's are host sizes of its CPU layout,
     // src/bcast_convolution.cpp:72-82).
@@ -497,6 +522,8 @@ void xnor_nn_destroy_convolution(xnor_nn_convolution_t *c) {
     if (st->stage_weights) (void)hipFree(st->stage_weights);
     if (st->stage_dst) (void)hipFree(st->stage_dst);
     if (st->float_parts) (void)hipFree(st->float_parts);
+    if (st->order_before) (void)hipEventDestroy(st->order_before);
+    if (st->order_after) (void)hipEventDestroy(st->order_after);
     drop_timer(st->time_binarize);
     drop_timer(st->time_convolution);
     delete st;
@@ -585,6 +612,13 @@ xnor_nn_status_t xnor_nn_hip_binarize_weights_float_noalloc(const xnor_nn_convol
                 "is %lld\n", n, (long long)XNOR_NN_HIP_NOALLOC_MAX_WEIGHTS);
         return xnor_nn_error_invalid_input;
     }
+    // hipPointerGetAttributes allocates nothing; a host pointer handed to the kernels would be
+    // a GPU memory fault
+    if (!on_device(from) || !on_device(to)) {
+        fprintf(stderr, "xnor_nn_hip_binarize_weights_float_noalloc: `from` and `to` must be "
+                "device pointers\n");
+        return xnor_nn_error_invalid_input;
+    }
     float *parts = nullptr;
     if (weights_float_scratch(&parts) != hipSuccess) {
         (void)hipGetLastError();
@@ -599,7 +633,14 @@ xnor_nn_status_t xnor_nn_hip_set_stream(const xnor_nn_convolution_t *c, void *st
     if (!bcast_descriptor(c)) return xnor_nn_error_invalid_input;
     State *st = state_of(c);
     std::lock_guard<std::mutex> call(st->mu);
-    st->stream = static_cast<hipStream_t>(stream);
+    hipStream_t to = static_cast<hipStream_t>(stream);
+    // xnor_nn_binarize_weights_float keeps its partial sums with the descriptor: kernels of an
+    // earlier call that are still under way on the old stream must be through with them
+    // before a call on the new stream may overwrite them
+    if (to != st->stream && st->float_parts != nullptr
+            && hipStreamSynchronize(st->stream) != hipSuccess)
+        return xnor_nn_error_memory;
+    st->stream = to;
     return xnor_nn_success;
 }
 
@@ -617,8 +658,11 @@ xnor_nn_status_t xnor_nn_hip_time_kernels(const xnor_nn_convolution_t *c, int ca
     State *st = state_of(c);
     std::lock_guard<std::mutex> call(st->mu);
     if (hipStreamSynchronize(st->stream) != hipSuccess) return xnor_nn_error_memory;
-    if (!make_timer(st->time_binarize, capacity) || !make_timer(st->time_convolution, capacity))
+    if (!make_timer(st->time_binarize, capacity) || !make_timer(st->time_convolution, capacity)) {
+        drop_timer(st->time_binarize); // never one stage timed and the other not
+        drop_timer(st->time_convolution);
         return xnor_nn_error_memory;
+    }
     return xnor_nn_success;
 }
 

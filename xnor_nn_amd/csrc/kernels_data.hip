@@ -384,17 +384,20 @@ bool nhwc_by_lane(const Geometry &g) {
 
 // The tiled kernel addresses the input with 32-bit byte offsets and stages the packed words
 // of a tile in LDS (64 KB at most: up to 8160 channels); deeper or larger inputs run the
-// generic kernel.
+// generic kernel.  A channel past the end of a ragged slice is read through the byte offset
+// 0xFFFFFFF0, which has to lie outside the buffer for the load to return +0: the input must
+// end below that offset.
 static bool tiled_nchw(const Geometry &g) {
     return g.src_fmt == xnor_nn_data_format_nchw
-        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull
+        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < XNOR_HIP_DROPPED_OFFSET
         && sizeof(uint32_t) * (TILE + (size_t)TILE * g.xw) <= 64 * 1024;
 }
 
-// The NHWC kernel reads 16 bytes per load at 32-bit byte offsets.
+// The NHWC kernel reads 16 bytes per load at 32-bit byte offsets (and drops pieces past the
+// last channel the same way).
 static bool vector_nhwc(const Geometry &g) {
     return g.src_fmt == xnor_nn_data_format_nhwc && (g.ic & 3) == 0
-        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < 0xFFFFFFFFull;
+        && (uint64_t)g.npix_in * (uint64_t)g.ic * 4u < XNOR_HIP_DROPPED_OFFSET;
 }
 
 const char *binarize_kernel_name(const Geometry &g) {

@@ -16,6 +16,11 @@
 
 #include "xnor_nn.h"
 
+// Byte offset that the kernels give a buffer access they want the hardware to drop (a channel
+// past the end, a dead pixel): it has to lie outside every buffer it is used with, so the
+// kernels that use it take buffers below this size only.
+#define XNOR_HIP_DROPPED_OFFSET 0xFFFFFFF0ull
+
 namespace xnor_hip {
 
 // n / d for 32-bit n by multiply-high and shifts; d is fixed on the host.
@@ -126,6 +131,9 @@ struct State {
     // convolution.  What is handed over is recorded per resource table, not here (api.hip).
     bool fuse_stages = true;
     bool verbose = false;
+    // Orders this descriptor's stream with another one (a box filter owed by a descriptor
+    // that runs on another stream); created on first use, under mu.
+    hipEvent_t order_before = nullptr, order_after = nullptr;
     KernelTimer time_binarize, time_convolution; // empty unless timing is switched on
 };
 
