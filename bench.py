@@ -15,6 +15,9 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+# the CPU baseline's OpenMP threads stay on neighbouring cores (set before any OpenMP runtime
+# starts; the GPU legs do not depend on it)
+os.environ.setdefault("OMP_PROC_BIND", "close")
 
 METRIC = "ms/forward + effective binary GOPS, AlexNet conv4 N=256 on 1 MI355X"
 HBM_PEAK_GBS = 8000.0
@@ -67,47 +70,70 @@ def work_figures(d):
     }
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(d, x, w, threads):
-    """The CPU path timed on this host: the compiled upstream library when it was built
-    (oracle/_ref), else the in-repo C restatement.  Baseline only; never the product."""
+    """The CPU path timed on this host, methodology of the reference's own benchmark
+    (reference test/perf/test_simple_net.cpp:39-60: per-stage timers around repeated forward
+    passes, minimum reported; the median is given beside it because this host is shared):
+    the compiled upstream library when it was built (oracle/_ref, kind "reference") and the
+    in-repo C restatement (oracle/, kind "port"), each on the whole workload, OpenMP on all
+    host threads with OMP_PROC_BIND=close.  Baselines only; never the product.  Returns
+    (headline entry, all entries): the reference when it is there, else the port."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import checkers
-    reps = 5 if d["mb"] * d["oc"] * d["ih"] * d["iw"] < 5e7 else 3
+    reps = 7 if d["mb"] * d["oc"] * d["ih"] * d["iw"] < 5e7 else 5
+    nominal = work_figures(d)["nominal_ops"]
+
+    def entry(kind, passes):
+        # passes: (t0, t1, t2, t3) per forward pass, the first one (warm-up) already dropped
+        totals = sorted(1e3 * (p[3] - p[0]) for p in passes)
+        best = min(passes, key=lambda p: p[3] - p[0])
+        stages = [1e3 * (best[i + 1] - best[i]) for i in range(3)]
+        ms, median = totals[0], totals[len(totals) // 2]
+        return {
+            "value": nominal / (ms * 1e-3) / 1e9, "unit": "GOPS",
+            "ms_per_forward": ms, "ms_per_forward_median": median,
+            "ms_per_forward_all": totals,
+            "value_at_median": nominal / (median * 1e-3) / 1e9,
+            "stage_ms": {"binarize_data": stages[0], "calculate_k": stages[1],
+                         "forward": stages[2]},
+            "cores": threads, "kind": kind, "cpu": cpu_model(),
+            "sample": "whole workload, minimum (and median) of %d forward passes after one "
+                      "warm-up (OpenMP, %d threads, OMP_PROC_BIND=%s%s)" % (
+                          len(passes), threads, os.environ.get("OMP_PROC_BIND", "unset"),
+                          ", XNOR_NN_ISA=2: AVX kernels" if kind == "reference" else ""),
+        }
+
+    entries = []
     if checkers.have_ref():
         ref = checkers.RefLib()
         out = ref.forward(d, x, w, reps=reps + 1, timer=time.perf_counter)
-        times = out["times"][1:]
-        best = min(times, key=lambda t: t[3] - t[0])
-        stages = [1e3 * (best[i + 1] - best[i]) for i in range(3)]
-        kind = "reference"
-    else:
-        from util import oracle_shape
-        oracle = checkers.Oracle()
-        s = oracle_shape(oracle, d)
-        bw, alpha, opc = oracle.binarize_weights(s, w)
-        best = None
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            bsrc = oracle.binarize_data(s, x)
-            t1 = time.perf_counter()
-            a, k = oracle.calculate_k(s, x)
-            t2 = time.perf_counter()
-            oracle.convolution(s, bsrc, bw, alpha, k, opc)
-            t3 = time.perf_counter()
-            if best is None or t3 - t0 < best[3] - best[0]:
-                best = (t0, t1, t2, t3)
-        stages = [1e3 * (best[i + 1] - best[i]) for i in range(3)]
-        kind = "port"
-    ms = sum(stages)
-    return {
-        "value": work_figures(d)["nominal_ops"] / (ms * 1e-3) / 1e9, "unit": "GOPS",
-        "ms_per_forward": ms, "stage_ms": {"binarize_data": stages[0],
-                                           "calculate_k": stages[1], "forward": stages[2]},
-        "cores": threads, "kind": kind,
-        "sample": "whole workload, best of %d forward passes after one warm-up "
-                  "(OpenMP, %d threads%s)" % (reps, threads,
-                                              ", XNOR_NN_ISA=2" if kind == "reference" else ""),
-    }
+        entries.append(entry("reference", out["times"][1:]))
+    from util import oracle_shape
+    oracle = checkers.Oracle()
+    s = oracle_shape(oracle, d)
+    bw, alpha, opc = oracle.binarize_weights(s, w)
+    passes = []
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        bsrc = oracle.binarize_data(s, x)
+        t1 = time.perf_counter()
+        a, k = oracle.calculate_k(s, x)
+        t2 = time.perf_counter()
+        oracle.convolution(s, bsrc, bw, alpha, k, opc)
+        t3 = time.perf_counter()
+        passes.append((t0, t1, t2, t3))
+    entries.append(entry("port", passes[1:]))
+    return entries[0], entries
 
 
 def main():
@@ -125,6 +151,10 @@ def main():
                     help="profiling aid: every step of the run, warm-up included, rotates "
                          "through the buffer pairs, so that a kernel trace of the run holds "
                          "cold launches only")
+    ap.add_argument("--binarize-only", action="store_true",
+                    help="profiling aid, with --cold-only: the rotation runs the binarize "
+                         "stage alone (no convolution output waiting in the caches to be "
+                         "written back while it reads)")
     ap.add_argument("--no-host", action="store_true",
                     help="skip the three forward passes through host buffers")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -167,6 +197,8 @@ def main():
         conv.stage("calculate_k")
         conv.stage("forward")
 
+    host_us = []  # host time per step of the three executor calls (enqueue only), per leg
+
     def timed_steps(sets):
         """K steps over the (input, output) pairs of `sets` in turn: wall clock per step, then
         the same K steps again with HIP events attached to every kernel launch (their own
@@ -176,6 +208,7 @@ def main():
         t0 = time.perf_counter()
         for i in range(args.steps):
             step(*sets[i % len(sets)])
+        host_us.append(1e6 * (time.perf_counter() - t0) / args.steps)  # all enqueued, none awaited
         torch.cuda.synchronize()
         wall_ms = 1e3 * (time.perf_counter() - t0) / args.steps
         conv.time_kernels(args.steps)
@@ -193,6 +226,14 @@ def main():
     if args.cold_only:
         sets = [(xt, yt)] + [(xt.clone(), torch.empty_like(yt)) for _ in range(nsets - 1)]
         torch.cuda.synchronize()
+        if args.binarize_only:
+            for i in range(max(args.warmup, nsets) + 2 * args.steps):
+                conv.stage("binarize_data", src=sets[i % nsets][0], dst=sets[i % nsets][1])
+            torch.cuda.synchronize()
+            print(json.dumps({"cold_only": True, "binarize_only": True,
+                              "workload": args.workload, "buffer_pairs": nsets}))
+            conv.close()
+            return
         for i in range(max(args.warmup, nsets)):
             step(*sets[i % nsets])
         cold_ms, cbin_ms, cconv_ms, _, _ = timed_steps(sets)
@@ -211,6 +252,7 @@ def main():
     # workload: they stay in the 256 MB Infinity Cache between steps).  The timed region is
     # exactly K steps, nothing but the three executor calls per step.
     ms_per_step, bin_ms, conv_ms, tb_sorted, tc_sorted = timed_steps([(xt, yt)])
+    warm_host_us = host_us[-1]
 
     # K launches of the binarize kernel alone, back to back, one pair of events around all
     region = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
@@ -312,9 +354,15 @@ def main():
                   "kernels' own dispatches; binarize_alone_us: K back-to-back launches "
                   "between two events; step_ms_between_events: one event between "
                   "consecutive steps; host_buffers_ms_per_forward: three passes through "
-                  "pageable host arrays",
+                  "pageable host arrays; host_enqueue_per_step: host time of the executor "
+                  "calls of a step (us), from the time to enqueue the K steps",
         "kernel_us": {"binarize": bin_ms * 1e3, "convolution": conv_ms * 1e3,
                       "step_minus_kernels": (ms_per_step - bin_ms - conv_ms) * 1e3,
+                      # what the host spends in the three executor calls of a step (pointer
+                      # queries, two mutexes, two launches), measured as the time to enqueue
+                      # the K steps; the rest of step_minus_kernels is the gap between
+                      # dependent dispatches on the GPU
+                      "host_enqueue_per_step": warm_host_us,
                       "binarize_alone": bin_alone_ms * 1e3,
                       "binarize_min_median_max": [tb_sorted[0] * 1e3,
                                                   tb_sorted[len(tb_sorted) // 2] * 1e3,
@@ -434,8 +482,9 @@ def main():
         result["copy_calibration_bytes_each_way"] = n * 4
     if not args.no_cpu:
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        cb = cpu_baseline(d, x, w, threads)
+        cb, both = cpu_baseline(d, x, w, threads)
         result["cpu_baseline"] = cb
+        result["cpu_baselines"] = both  # the real reference and the in-repo restatement
         result["speedup_vs_cpu_baseline"] = cb["ms_per_forward"] / ms_per_step
     print(json.dumps(result))
 
