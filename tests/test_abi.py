@@ -244,10 +244,13 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     boundary shapes get, decided at init from the shape alone."""
     for key in ("XNOR_NN_HIP_CONV", "XNOR_NN_HIP_MFMA_PS", "XNOR_NN_HIP_MFMA_MIX",
                 "XNOR_NN_HIP_MFMA_PAIR", "XNOR_NN_HIP_NHWC", "XNOR_NN_HIP_STREAM_DST",
-                "XNOR_NN_HIP_MFMA_PERSIST"):
+                "XNOR_NN_HIP_MFMA_PERSIST", "XNOR_NN_HIP_MFMA_SMALL"):
         monkeypatch.delenv(key, raising=False)
     conv4 = (256, 384, 13, 13, 3, 3, 1, 1, 1, 1)
-    assert kernel_names((1,) + conv4) == ("binarize_nchw_kernel", "conv_mfma_fp4_kernel<KS=6,PS=1>")
+    # 6 pixel blocks x 8 filter blocks: fewer (block, block) pairs than compute units
+    assert kernel_names((1,) + conv4) == ("binarize_nchw_kernel", "conv_mfma_fp4_small_kernel<KS=6>")
+    assert kernel_names((8,) + conv4)[1] == "conv_mfma_fp4_small_kernel<KS=6>"
+    assert kernel_names((16,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=1>"
     # 5.3 pixel blocks per compute unit: two tile sizes in one launch
     assert kernel_names((256,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4+2>"
     assert kernel_names((1024,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4>"

@@ -806,3 +806,35 @@ def test_persistent_workgroups(oracle, monkeypatch, t, fmts, wgs):
     if wgs >= chunks:
         assert name.startswith("conv_mfma_fp4_persistent_kernel"), name
     run_and_compare(oracle, d, xs, ws, fmts)
+
+
+@pytest.mark.parametrize("separate_k", [False, True], ids=["fused_k", "k_plane"])
+@pytest.mark.parametrize("t,fmts", [
+    ((1, 256, 384, 13, 13, 3, 3, 1, 1, 1, 1), NCHW),                     # conv4, minibatch 1
+    ((3, 100, 70, 9, 7, 3, 3, 1, 1, 1, 1), NCHW),                        # ragged filters, channels, pixels
+    ((2, 64, 64, 28, 28, 3, 3, 2, 2, 1, 1), (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC)),
+    ((1, 512, 33, 14, 14, 1, 1, 1, 1, 0, 0), NCHW),                      # one tap, eight steps
+    ((2, 40, 128, 6, 5, 5, 5, 1, 1, 2, 2), (capi.FMT_NHWC, capi.FMT_HWIO, capi.FMT_NCHW)),
+    ((1, 1000, 16, 4, 4, 3, 3, 1, 1, 1, 1), NCHW),                       # sixteen steps per tap
+    ((1, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0), NCHW),                           # the smallest problem
+    ((5, 600, 64, 3, 3, 7, 7, 4, 4, 3, 3), NCHW),                        # kernel wider than the image
+], ids=lambda v: shapes.shape_id(v) if len(v) == 11 else "fmt%d%d%d" % v)
+def test_small_problem_kernel(oracle, monkeypatch, t, fmts, separate_k):
+    """The matrix-core kernel for launches of few tiles (a workgroup per 32 pixels x 32 filters,
+    the four waves splitting the taps and adding their exact partial sums through LDS; chosen
+    by size at init, conv4 at minibatch 1 takes it), forced on here for ragged and odd shapes,
+    with K summed in the kernel and with K read from the plane."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_SMALL", "1")
+    if separate_k:
+        monkeypatch.setenv("XNOR_NN_HIP_SEPARATE_K", "1")
+    d = shapes.as_dims(t)
+    x = synth.normal(171, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::5] = 0.0
+    w = synth.normal(172, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    xs = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if fmts[0] == capi.FMT_NHWC else x
+    ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
+    name = make(d, ws, fmts).kernel_name(0)
+    assert name.startswith("conv_mfma_fp4_small_kernel"), name
+    run_and_compare(oracle, d, xs, ws, fmts)

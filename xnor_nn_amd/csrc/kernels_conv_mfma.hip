@@ -61,26 +61,6 @@ constexpr int MAX_DEVICES = 64;
 // faster (AlexNet conv4 MB 256: this kernel 23.6 us against 28.8 us streaming).
 constexpr int STORE_WRITE_BACK = 0, STORE_STREAMING = 2;
 
-// First and last input pixel (flattened index) that a tile of the output pixels
-// [p_first, p_end) can touch with an in-bounds tap: from the start of the first input row of
-// its first pixel to the end of the last input row of its last pixel (with a stride above 1
-// the span also holds the input pixels the stride skips).
-__host__ __device__ inline void tile_span(const Geometry &g, uint32_t p_first, uint32_t p_end,
-        int &lo, int &hi) {
-    const uint32_t p_last = p_end - 1;
-    const uint32_t i0 = g.div_ohw.div(p_first), i1 = g.div_ohw.div(p_last);
-    const int oh0 = (int)g.div_ow.div(p_first - i0 * g.ohw);
-    const int oh1 = (int)g.div_ow.div(p_last - i1 * g.ohw);
-    int r0 = oh0 * g.sh - g.ph, r1 = oh1 * g.sh - g.ph + g.kh - 1;
-    if (r0 < 0) r0 = 0;
-    if (r0 > g.ih - 1) r0 = g.ih - 1;
-    if (r1 > g.ih - 1) r1 = g.ih - 1;
-    if (r1 < 0) r1 = 0;
-    lo = (int)(i0 * g.ihw) + r0 * g.iw;
-    hi = (int)(i1 * g.ihw) + r1 * g.iw + g.iw - 1;
-    if (hi < lo) hi = lo;
-}
-
 __device__ __forceinline__ v16f mfma_fp4(const v4i a, const v4i b, const v16f c) {
     const v8i a8 = {a.x, a.y, a.z, a.w, 0, 0, 0, 0};
     const v8i b8 = {b.x, b.y, b.z, b.w, 0, 0, 0, 0};
@@ -1367,6 +1347,8 @@ void mfma_plan(Geometry &g) {
     g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
     g.mfma_ps_small = 0;
     g.mfma_big_per_xcd = g.mfma_blocks_per_xcd = 0;
+    g.mfma_small = g.mfma_small_rows = 0;
+    g.mfma_small_lds = 0;
     g.mfma_persist = g.mfma_reverse = 0;
     g.mfma_tiles_per_round = g.mfma_rounds = g.mfma_stagger = 0;
     g.stream_dst = 0;
@@ -1390,6 +1372,17 @@ void mfma_plan(Geometry &g) {
     g.mfma_rows = max_tile_rows(g, 32 * g.mfma_ps);
     g.mfma_lds = (uint32_t)lds_bytes(g, g.mfma_ps);
     g.mfma_wbytes = (uint32_t)mfma_weight_bytes(g);
+    // Few tiles: the small-problem kernel takes the scaled output (the raw accumulators still
+    // go through the kernel planned below).
+    {
+        int rows = 0;
+        uint32_t lds = 0;
+        if (small_kernel_applies(g, &rows, &lds)) {
+            g.mfma_small = 1;
+            g.mfma_small_rows = rows;
+            g.mfma_small_lds = lds;
+        }
+    }
     // Two tile sizes in one launch (see the kernel): worth it when every compute unit gets
     // more than four and at most six pixel blocks, i.e. when equal tiles would give it two
     // workgroups of three that finish together.  Needs the four-block variant and room for
@@ -1499,7 +1492,9 @@ hipError_t launch_pack_weights_fp4(const Geometry &g, const float *w, uint32_t *
 
 const char *mfma_kernel_name(const Geometry &g) {
     static thread_local char name[80];
-    if (g.mfma_parts > 1)
+    if (g.mfma_small)
+        snprintf(name, sizeof name, "conv_mfma_fp4_small_kernel<KS=%d>", g.mfma_steps);
+    else if (g.mfma_parts > 1)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d,PARTS=%d>",
                 g.mfma_steps, g.mfma_ps, g.mfma_parts);
     else if (g.mfma_persist)
@@ -1517,6 +1512,8 @@ const char *mfma_kernel_name(const Geometry &g) {
 hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
         const uint32_t *wfrag, const float *alpha, const float *k,
         float *dst, int32_t *popc, const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
+    if (g.mfma_small && popc == nullptr)
+        return launch_convolution_small(g, xbits, wfrag, alpha, k, dst, a_or_null, k_out, s, ev);
     if (g.mfma_pair) {
         switch (g.xw) {
         case 1: return launch_mfma_ps<1, true>(g, xbits, wfrag, alpha, k, dst, popc, a_or_null, k_out, s, ev);

@@ -82,10 +82,33 @@ struct Geometry {
     // per pair of taps), tap pairing, channel parts, input pixels a tile stages at most, LDS
     // bytes per workgroup, bytes of the weight fragments
     int mfma_steps, mfma_pair, mfma_parts, mfma_rows;
+    int mfma_small;             // 1: few tiles: the small-problem kernel (kernels_conv_small.hip),
+    int mfma_small_rows;        // the input pixels one of its blocks stages at most
+    uint32_t mfma_small_lds;    // and its LDS bytes per workgroup
     int stream_dst;             // 1: the matrix-core kernel stores its output with the nt bit
     uint32_t mfma_lds, mfma_wbytes;
     FastDiv div_ihw, div_iw, div_ohw, div_ow;
 };
+
+// First and last input pixel (flattened index) that a tile of the output pixels
+// [p_first, p_end) can touch with an in-bounds tap: from the start of the first input row of
+// its first pixel to the end of the last input row of its last pixel (with a stride above 1
+// the span also holds the input pixels the stride skips).
+__host__ __device__ inline void tile_span(const Geometry &g, uint32_t p_first, uint32_t p_end,
+        int &lo, int &hi) {
+    const uint32_t p_last = p_end - 1;
+    const uint32_t i0 = g.div_ohw.div(p_first), i1 = g.div_ohw.div(p_last);
+    const int oh0 = (int)g.div_ow.div(p_first - i0 * g.ohw);
+    const int oh1 = (int)g.div_ow.div(p_last - i1 * g.ohw);
+    int r0 = oh0 * g.sh - g.ph, r1 = oh1 * g.sh - g.ph + g.kh - 1;
+    if (r0 < 0) r0 = 0;
+    if (r0 > g.ih - 1) r0 = g.ih - 1;
+    if (r1 > g.ih - 1) r1 = g.ih - 1;
+    if (r1 < 0) r1 = 0;
+    lo = (int)(i0 * g.ihw) + r0 * g.iw;
+    hi = (int)(i1 * g.ihw) + r1 * g.iw + g.iw - 1;
+    if (hi < lo) hi = lo;
+}
 
 // Optional timing of one launch: when both events are set the kernel is launched with them
 // attached to its own dispatch, and their difference is the kernel's duration on the GPU (no
@@ -179,6 +202,12 @@ hipError_t launch_convolution_mfma(const Geometry &g, const uint32_t *xbits,
 // (32x32x64) on register-resident +-1 operands
 hipError_t launch_mfma_only(int workgroups, int iterations, hipStream_t s);
 const char *convolution_kernel_name(const Geometry &g);
+// The matrix-core kernel for launches of few tiles (filled in by mfma_plan: g.mfma_small).
+bool small_kernel_applies(const Geometry &g, int *rows, uint32_t *lds);
+hipError_t launch_convolution_small(const Geometry &g, const uint32_t *xbits,
+        const uint32_t *wfrag, const float *alpha, const float *k, float *dst,
+        const float *a_or_null, float *k_out, hipStream_t s,
+        const KernelEvents &ev = KernelEvents{});
 const char *binarize_kernel_name(const Geometry &g);
 
 int pick_q(int oc, int xw);
