@@ -669,11 +669,13 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
     images up to 43 x 43, every layout combination, inputs with exact zeros of both signs;
     every third problem with a two-tile-size launch forced on (four and two, four and three),
     every third with persistent workgroups forced on (one to three per XCD, so that each walks
-    over many tiles), every fourth with streaming output stores): dst and the raw popcounts against the oracle, bit for bit, stopping at
-    the first mismatch."""
+    over many tiles), every sixth with the small-problem kernel forced on wherever it can run,
+    every fourth with streaming output stores): dst and the raw popcounts against the oracle,
+    bit for bit, stopping at the first mismatch.  XNOR_NN_TEST_RANDOM_SECONDS and
+    XNOR_NN_TEST_RANDOM_SEED lengthen the run and move it to other problems."""
     import time
-    rng = np.random.default_rng(20251)
-    t_end = time.time() + 15.0
+    rng = np.random.default_rng(int(os.environ.get("XNOR_NN_TEST_RANDOM_SEED", "20251")))
+    t_end = time.time() + float(os.environ.get("XNOR_NN_TEST_RANDOM_SECONDS", "15"))
     n = 0
     while time.time() < t_end:
         kh, kw = int(rng.integers(1, 10)), int(rng.integers(1, 10))
@@ -707,6 +709,7 @@ def test_random_problems_until_the_time_is_up(oracle, monkeypatch):
         # launch options that the library otherwise picks by problem size
         forced = {"XNOR_NN_HIP_MFMA_MIX": "1" if n % 6 == 2 else "3" if n % 6 == 5 else None,
                   "XNOR_NN_HIP_MFMA_PERSIST": str(1 + n % 3) if n % 6 in (0, 3) else None,
+                  "XNOR_NN_HIP_MFMA_SMALL": "1" if n % 6 == 1 else None,
                   "XNOR_NN_HIP_STREAM_DST": "1" if n % 4 == 3 else None}
         for key, value in forced.items():
             if value is None:
