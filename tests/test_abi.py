@@ -254,11 +254,15 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     # 5.3 pixel blocks per compute unit: two tile sizes in one launch
     assert kernel_names((256,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4+2>"
     assert kernel_names((1024,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4>"
-    # 96 channels = three words: two taps share three steps
+    # 96 channels = three words: two taps share three steps; several rounds of tiles with at
+    # most four steps per tap: tiles of two blocks, three workgroups to a compute unit
     assert kernel_names((128, 256, 96, 27, 27, 5, 5, 1, 1, 2, 2))[1] \
-        == "conv_mfma_fp4_kernel<KS=3,PS=4,PAIR>"
+        == "conv_mfma_fp4_kernel<KS=3,PS=2,PAIR>"
     assert kernel_names((64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
-        == "conv_mfma_fp4_kernel<KS=4,PS=4>"
+        == "conv_mfma_fp4_kernel<KS=4,PS=2>"
+    # 64 filters: one wave of four has work, the slots of a compute unit count all the same
+    assert kernel_names((64, 64, 64, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
+        == "conv_mfma_fp4_kernel<KS=1,PS=2>"
     # 98 blocks for 32 slots per XCD and filter chunk: 2 tiles of four, 30 of three
     assert kernel_names((32, 512, 512, 28, 28, 3, 3, 1, 1, 1, 1))[1] \
         == "conv_mfma_fp4_kernel<KS=8,PS=4+3>"
@@ -300,7 +304,7 @@ def test_persistent_workgroups_are_planned_on_request_only(monkeypatch):
     workgroup per tile, whatever the size (measured faster)."""
     resnet = (64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1)
     monkeypatch.delenv("XNOR_NN_HIP_MFMA_PERSIST", raising=False)
-    assert kernel_names(resnet)[1] == "conv_mfma_fp4_kernel<KS=4,PS=4>"
+    assert kernel_names(resnet)[1] == "conv_mfma_fp4_kernel<KS=4,PS=2>"
     monkeypatch.setenv("XNOR_NN_HIP_MFMA_PERSIST", "64")
     assert kernel_names(resnet)[1] == "conv_mfma_fp4_persistent_kernel<KS=4,PS=4+3>"
     # sixteen steps per tap have no four-block tile: never persistent

@@ -216,10 +216,16 @@ def by_hand(*lines):
     return [ASM_BEGIN] + list(lines) + [ASM_END]
 
 
-def test_no_register_is_touched_while_its_load_is_in_flight(tmp_path):
+@pytest.fixture(scope="module")
+def conv_isa(tmp_path_factory):
+    """The matrix-core kernels as the compiler prints them (one compilation for the module)."""
+    return compile_to_isa(tmp_path_factory.mktemp("isa"), "kernels_conv_mfma")
+
+
+def test_no_register_is_touched_while_its_load_is_in_flight(conv_isa):
     """Every variant of the matrix-core kernel that the library holds (all of them can be
     launched), from its first instruction to the end."""
-    isa = compile_to_isa(tmp_path, "kernels_conv_mfma")
+    isa = conv_isa
     checked = 0
     for name, body in kernels_of(isa, r"^_ZN\S*conv_mfma_fp4\S*kernel\S*:"):
         lines = instructions(body)
@@ -313,3 +319,45 @@ def test_lds_direct_loads_count_but_write_no_register():
     assert hazards_of(ok) == []
     assert m0_outside_asm(ok) == []
     assert m0_outside_asm(ok + ["s_mov_b32 m0, s8"]) == ["s_mov_b32 m0, s8"]
+
+
+def resident_by_registers(ks, ps):
+    """The register half of resident_workgroups() in kernels_conv_mfma.hip, restated."""
+    if ps == 3:
+        return 3 if ks == 1 else 2
+    if ps == 2:
+        return 4 if ks == 1 else 3 if (ks <= 4 or ks == 12) else 2
+    if ps == 1:
+        return 4 if (ks <= 4 or ks >= 12) else 3 if ks <= 6 else 2
+    return 2
+
+
+def test_the_tile_model_counts_resident_workgroups_as_the_registers_allow(conv_isa):
+    """The tile-size model prices a tile by how many workgroups fit a compute unit together.
+    Its register rule is held against the compiler's own counts (.vgpr_count of the kernel
+    metadata, 512 registers per SIMD lane in granules of 8) for every forward variant with
+    one tile size: the rule never promises a workgroup that does not fit, and is exact for all
+    but a few variants."""
+    counts, name = {}, None
+    for line in conv_isa:
+        line = line.strip()
+        if line.startswith(".name:"):
+            name = line.split()[1]
+        elif line.startswith(".vgpr_count:") and name:
+            counts[name] = int(line.split()[1])
+    plain = subprocess.run(["c++filt"], input="\n".join(counts), capture_output=True, text=True,
+                           check=True).stdout.split("\n")
+    seen = exact = 0
+    for mangled, text in zip(counts, plain):
+        m = re.search(r"conv_mfma_fp4_kernel<(\d+), (\d+), (\d+), (\w+), (\w+), (\w+)>", text)
+        if not m or m[3] != "0" or m[4] == "true":  # two tile sizes, raw accumulators
+            continue
+        ks, ps = int(m[1]), int(m[2])
+        fit = min(4, 512 // ((counts[mangled] + 7) // 8 * 8))
+        rule = resident_by_registers(ks, ps)
+        assert rule <= fit, "%s: %d registers hold %d workgroups, the model counts %d" % (
+            text[:60], counts[mangled], fit, rule)
+        seen += 1
+        exact += rule == fit
+    assert seen >= 40, seen
+    assert seen - exact <= 2, (seen, exact)

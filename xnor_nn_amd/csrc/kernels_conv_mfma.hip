@@ -1150,18 +1150,45 @@ size_t lds_bytes(const Geometry &g, int ps) {
 //               -- with one pixel block and more than one wave per SIMD a step costs as much
 //               as with two: the weight stream (2 KB per wave and step whatever the tile)
 //               sets its pace, not the matrix instructions;
+//               Tiles of two pixel blocks pay 10 % more per step: their weight stream is
+//               as wide as the vector-memory return path of the CU;
 //   the kernel: one wave's time for the first wave of the busiest SIMD, 0.35 of it more for
-//               the second (the phases of two resident waves overlap), 0.75 for every further
-//               one; with few waves per SIMD the busiest one counts (rounded up), with many
-//               the hardware's dynamic scheduling evens the load out;
+//               every further wave that is resident with it (their phases overlap), and for
+//               every wave beyond the resident ones 0.75 of it with two resident waves per
+//               SIMD, 0.5 with three, 0.35 with four (small tiles of shallow inputs need at
+//               most 168 or 128 registers, so a third or fourth workgroup fits a CU, and a
+//               launch of many rounds of such tiles is faster than one of large tiles:
+//               ResNet 3x3 56x56 MB 64 61.0 against 63.1 us, 128 filters on the same input
+//               32.5 against 38.1, 64 filters 18.0 against 23.5); with few waves per SIMD the
+//               busiest one counts (rounded up), with many the hardware's dynamic
+//               scheduling evens the load out;
 //   a tile that needs more than half the LDS runs alone on its CU: 15 % more.
 // Ties go to the larger tile, which streams fewer weight bytes.
+// Refitted on 56 shapes (13x13 to 112x112 images, 32 to 512 channels, 64 to 512 filters,
+// 1x1 to 5x5 kernels, MB 1 to 1024) with every tile size forced in turn: the choice is the
+// fastest tile on 50 of them and within 3.2 % on the rest.
 // Four pixel blocks do not fit the register file with 16 steps per tap or with tap pairing
 // over five words (those variants spill), and are not instantiated for channel parts.
 bool tile_fits_registers(const Geometry &g, int ps) {
     if (ps < 4) return true;
     if (channel_parts(g) > 1) return false;
     return pair_taps(g) ? g.xw < 5 : steps_per_tap(g) < 16;
+}
+
+// Workgroups of a tile size that fit a compute unit together, two to four: by registers (the
+// counts of the compiled variants: four pixel blocks 199 to 254, three 168 with one step per
+// tap and 184 or more otherwise, two 119 with one step per tap, 135 to 167 with two to four or
+// twelve steps and 188 or more otherwise, one 70 to 118 up to four steps and from twelve, 139
+// or 149 with five or six, 181 with eight; a SIMD holds 512 per lane) and by LDS.
+int resident_workgroups(const Geometry &g, int ps) {
+    const int ks = steps_per_tap(g);
+    int by_regs = 2;
+    if (ps == 3) by_regs = ks == 1 ? 3 : 2;
+    if (ps == 2) by_regs = ks == 1 ? 4 : (ks <= 4 || ks == 12) ? 3 : 2;
+    if (ps == 1) by_regs = (ks <= 4 || ks >= 12) ? 4 : ks <= 6 ? 3 : 2;
+    const int by_lds = (int)((size_t)LDS_LIMIT / lds_bytes(g, ps));
+    const int fit = by_regs < by_lds ? by_regs : by_lds;
+    return fit < 2 ? 2 : fit; // a tile that runs alone is priced separately
 }
 
 int pick_ps(const Geometry &g) {
@@ -1171,7 +1198,6 @@ int pick_ps(const Geometry &g) {
             return v;
     }
     const int chunks = (g.oc + NT - 1) / NT;
-    const int waves_per_block = g.oc >= NT ? 4 : (g.oc + 63) / 64;
     const double simds = (double)g.cus * 4;
     const int units = pair_taps(g) ? (g.kh * g.kw + 1) / 2 : g.kh * g.kw * channel_parts(g);
     const double steps_total = (double)units * steps_per_tap(g);
@@ -1181,14 +1207,20 @@ int pick_ps(const Geometry &g) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
         if (!tile_fits_registers(g, ps)) continue;
         const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
-        const double per_simd = tiles * chunks * waves_per_block / simds;
+        // workgroups per compute unit = waves per SIMD; a workgroup whose filters fill fewer
+        // than four waves (OC below 256) still takes its slot with all four
+        const double per_simd = tiles * chunks * 4 / simds;
         const double busiest = per_simd <= 1 ? 1.0
             : per_simd <= 4 ? (double)(long)(per_simd + 0.999999) : per_simd + 0.5;
         const double words = (double)max_tile_rows(g, 32 * ps) * g.xw;
         const double stream_bound = ps < 2 && per_simd > 1 ? 2.0 : (double)ps;
         const double wave = 3700.0 + 264.0 * words / 256.0 + 1700.0 * ps
-            + 64.0 * steps_total * stream_bound;
-        const double waves = busiest < 2 ? 1.0 : 1.35 + 0.75 * (busiest - 2.0);
+            + (ps == 2 ? 70.4 : 64.0) * steps_total * stream_bound;
+        const int resident = resident_workgroups(g, ps);
+        const double further = resident >= 4 ? 0.35 : resident == 3 ? 0.5 : 0.75;
+        const double together = busiest < resident ? busiest : (double)resident;
+        const double waves = busiest < 2 ? 1.0
+            : 1.0 + 0.35 * (together - 1.0) + further * (busiest - together);
         const double alone = lds_bytes(g, ps) > (size_t)LDS_TWO_PER_CU ? 1.15 : 1.0;
         const double cost = wave * waves * alone;
         if (best == 0 || cost < best_cost - 1e-9) { best = ps; best_cost = cost; }
