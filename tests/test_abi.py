@@ -244,7 +244,7 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     boundary shapes get, decided at init from the shape alone."""
     for key in ("XNOR_NN_HIP_CONV", "XNOR_NN_HIP_MFMA_PS", "XNOR_NN_HIP_MFMA_MIX",
                 "XNOR_NN_HIP_MFMA_PAIR", "XNOR_NN_HIP_NHWC", "XNOR_NN_HIP_STREAM_DST",
-                "XNOR_NN_HIP_MFMA_PERSIST", "XNOR_NN_HIP_MFMA_SMALL"):
+                "XNOR_NN_HIP_MFMA_PERSIST", "XNOR_NN_HIP_MFMA_SMALL", "XNOR_NN_HIP_MFMA_GROUPS"):
         monkeypatch.delenv(key, raising=False)
     conv4 = (256, 384, 13, 13, 3, 3, 1, 1, 1, 1)
     # 6 pixel blocks x 8 filter blocks: fewer (block, block) pairs than compute units
@@ -260,9 +260,12 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
         == "conv_mfma_fp4_kernel<KS=3,PS=2,PAIR>"
     assert kernel_names((64, 256, 256, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
         == "conv_mfma_fp4_kernel<KS=4,PS=2>"
-    # 64 filters: one wave of four has work, the slots of a compute unit count all the same
+    # 64 filters are one wave's worth: the other three waves take further pixel blocks; 128
+    # filters: two pixel groups
     assert kernel_names((64, 64, 64, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
-        == "conv_mfma_fp4_kernel<KS=1,PS=2>"
+        == "conv_mfma_fp4_kernel<KS=1,PS=2,GROUPS=4>"
+    assert kernel_names((64, 128, 128, 56, 56, 3, 3, 1, 1, 1, 1))[1] \
+        == "conv_mfma_fp4_kernel<KS=2,PS=2,GROUPS=2>"
     # 98 blocks for 32 slots per XCD and filter chunk: 2 tiles of four, 30 of three
     assert kernel_names((32, 512, 512, 28, 28, 3, 3, 1, 1, 1, 1))[1] \
         == "conv_mfma_fp4_kernel<KS=8,PS=4+3>"

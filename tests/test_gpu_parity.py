@@ -196,7 +196,7 @@ def test_matrix_core_tile_sizes(oracle, gpu, monkeypatch, ps):
         d["mb"], d["ic"], d["ih"], d["iw"])
     w = synth.normal(76, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
         d["oc"], d["ic"], d["kh"], d["kw"])
-    assert make(d, w).kernel_name(0) == "conv_mfma_fp4_kernel<KS=12,PS=%s>" % ps
+    assert make(d, w).kernel_name(0) == "conv_mfma_fp4_kernel<KS=12,PS=%s,GROUPS=2>" % ps  # 70 filters
     run_and_compare(oracle, d, x, w)
 
 
@@ -218,7 +218,7 @@ def test_tap_pairing(oracle, monkeypatch, t, pair):
     w = synth.normal(72, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
         d["oc"], d["ic"], d["kh"], d["kw"])
     name = make(d, w).kernel_name(0)
-    assert name.startswith("conv_mfma") and name.endswith(",PAIR>") == (pair == "1"), name
+    assert name.startswith("conv_mfma") and (",PAIR" in name) == (pair == "1"), name
     run_and_compare(oracle, d, x, w)
 
 
@@ -841,3 +841,43 @@ def test_small_problem_kernel(oracle, monkeypatch, t, fmts, separate_k):
     name = make(d, ws, fmts).kernel_name(0)
     assert name.startswith("conv_mfma_fp4_small_kernel"), name
     run_and_compare(oracle, d, xs, ws, fmts)
+
+
+@pytest.mark.parametrize("separate_k", [False, True], ids=["fused_k", "k_plane"])
+@pytest.mark.parametrize("ps", ["1", "2", "3", "4"])
+@pytest.mark.parametrize("t,fmts,groups", [
+    ((3, 64, 64, 20, 20, 3, 3, 1, 1, 1, 1), NCHW, 4),                    # one wave's filters
+    ((2, 100, 33, 17, 13, 3, 3, 1, 1, 1, 1), NCHW, 4),                   # ragged everything
+    ((2, 96, 128, 15, 15, 5, 5, 1, 1, 2, 2), NCHW, 2),                   # tap pairs, two waves' filters
+    ((3, 128, 100, 14, 14, 3, 3, 2, 2, 1, 1), (capi.FMT_NCHW, capi.FMT_OIHW, capi.FMT_NHWC), 2),
+    ((2, 40, 64, 12, 11, 3, 3, 1, 1, 1, 1), (capi.FMT_NHWC, capi.FMT_HWIO, capi.FMT_NHWC), 4),
+    ((1, 256, 7, 23, 9, 1, 1, 1, 1, 0, 0), NCHW, 4),                     # 1x1, seven filters
+    ((5, 32, 65, 9, 9, 3, 3, 1, 1, 1, 1), NCHW, 2),                      # one filter in the second wave
+    ((1, 64, 16, 5, 5, 3, 3, 1, 1, 1, 1), NCHW, 4),                      # one block: three groups past the end
+], ids=lambda v: shapes.shape_id(v) if isinstance(v, tuple) and len(v) == 11
+   else "fmt%d%d%d" % v if isinstance(v, tuple) else "groups%d" % v)
+def test_pixel_groups_for_few_filters(oracle, monkeypatch, t, fmts, groups, ps, separate_k):
+    """With 128 filters or fewer the waves of a workgroup that would have no filters take the
+    same filters on further pixel blocks (two or four pixel groups per tile): every tile size,
+    ragged filter counts, both output layouts, strides, tap pairs, K summed in the kernel and
+    read from its plane, tiles whose later groups lie past the last pixel; and the same
+    problems with the groups switched off."""
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_SMALL", "0")
+    monkeypatch.setenv("XNOR_NN_HIP_MFMA_PS", ps)
+    if separate_k:
+        monkeypatch.setenv("XNOR_NN_HIP_SEPARATE_K", "1")
+    d = shapes.as_dims(t)
+    x = synth.normal(271, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+        d["mb"], d["ic"], d["ih"], d["iw"])
+    x.ravel()[::5] = 0.0
+    w = synth.normal(272, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+        d["oc"], d["ic"], d["kh"], d["kw"])
+    xs = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if fmts[0] == capi.FMT_NHWC else x
+    ws = np.ascontiguousarray(w.transpose(2, 3, 1, 0)) if fmts[1] == capi.FMT_HWIO else w
+    name = make(d, ws, fmts).kernel_name(0)
+    assert name.endswith("PS=%s%s,GROUPS=%d>" % (ps, ",PAIR" if "PAIR" in name else "", groups)), name
+    run_and_compare(oracle, d, xs, ws, fmts)
+    if not separate_k and ps == "2":
+        monkeypatch.setenv("XNOR_NN_HIP_MFMA_GROUPS", "1")
+        assert "GROUPS" not in make(d, ws, fmts).kernel_name(0)
+        run_and_compare(oracle, d, xs, ws, fmts)

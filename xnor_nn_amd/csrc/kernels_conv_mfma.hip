@@ -204,6 +204,10 @@ __device__ __forceinline__ void copy_to_lds_async(const void *src, const int n,
 // 32*KS bytes further into the same LDS rows.
 // One tile: the output pixels [p_first, min(p_first + 32*PS, p_limit)) x the 256 filters of
 // filter chunk `chunk`.
+// With 128 filters or fewer (g.mfma_groups = 2 or 4) the waves that would have no filters take
+// further pixels instead: the tile is 32*PS*groups pixels, wave w multiplies the filters of
+// wave w % (4/groups) with the pixel blocks of group w / (4/groups), and everything the
+// workgroup does together (staging, the K sums, the alphas) covers the whole tile.
 // PERSIST: the caller loops over tiles (see conv_mfma_fp4_persistent_kernel); `turn` says what
 // is already in LDS and which tile to prefetch.  The LDS layout then has room for four pixel
 // blocks whatever PS is, so that tiles of two sizes can follow each other.
@@ -240,8 +244,9 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     // NHWC output: per wave 32 pixel rows of TURN_ROW floats to turn a block around in
     // (an offset from smem, not a rounded pointer: the compiler has to see an LDS address)
     constexpr int PSL = PERSIST ? 4 : PS; // pixel blocks the layout has room for
+    const int groups = PERSIST ? 1 : g.mfma_groups; // pixel groups: 1, 2 or 4 (uniform)
     float *turn_lds = reinterpret_cast<float *>(smem + ((stage_at + stage_bytes
-            + (1 + max_rows) * ROW_BYTES + (max_rows + 1 + 32 * PSL) * 4 + 15) & ~15));
+            + (1 + max_rows) * ROW_BYTES + (max_rows + 1 + 32 * PSL * groups) * 4 + 15) & ~15));
     constexpr int MT = 32 * PS;
     // Weight fragments are fetched in groups of HS steps, one group ahead: a whole tap where
     // the registers allow it (8 VGPRs per step on top of 32 per pixel block), half a tap
@@ -260,12 +265,16 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     const int tid = thread;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // this wave's filters are those of wave `fw` of a full workgroup, its pixels those of
+    // pixel group `pg` (fw = wave, pg = 0 with one group)
+    const int nfw = 4 / groups, fw = wave & (nfw - 1), pg = wave / nfw;
+    const uint32_t p_wave = p_first + (uint32_t)(pg * MT);
     // "taps" below are the units the main loop walks over: kernel taps, or pairs of them
     const int taps = PAIR ? (g.kh * g.kw + 1) / 2 : DEEP ? g.kh * g.kw * ic_parts : g.kh * g.kw;
 
     // ---- which input pixels does the tile touch ------------------------------------------
     int lo, hi;
-    tile_span(g, p_first, min(p_first + (uint32_t)MT, p_limit), lo, hi);
+    tile_span(g, p_first, min(p_first + (uint32_t)(MT * groups), p_limit), lo, hi);
     const int nrows = min(hi - lo + 1, max_rows);
 
     // ---- the 32*PS output pixels of the tile, one per lane and 32-pixel block -----------------
@@ -277,7 +286,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     uint32_t pix[PS], img[PS], rem[PS];
 #pragma unroll
     for (int ps = 0; ps < PS; ps++) {
-        pix[ps] = p_first + ps * 32 + (lane & 31);
+        pix[ps] = p_wave + ps * 32 + (lane & 31);
         live[ps] = pix[ps] < p_limit;
         const uint32_t pc = live[ps] ? pix[ps] : p_limit - 1;
         img[ps] = g.div_ohw.div(pc);
@@ -379,14 +388,14 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
             if (i < nitems) expand(i, early[u]);
         }
     }
-    // K of the tile's pixels, when it is not read from the K plane: wave ps sums the block
-    // of 32 pixels ps exactly as the box filter does (in-bounds taps in row-major order, each
+    // K of the tile's pixels, when it is not read from the K plane: wave ps (of the waves
+    // that share a pixel group) sums the block of 32 pixels ps exactly as the box filter does (in-bounds taps in row-major order, each
     // product rounded, then added: reference src/bcast_calculate_k.cpp:69-85), leaves it in
     // LDS for the epilogue of all waves and stores it to the K plane.
     if (fuse_k) {
 #pragma unroll
         for (int ps = 0; ps < PS; ps++) {
-            if (ps != wave) continue; // uniform
+            if ((ps & (nfw - 1)) != fw) continue; // uniform
             float sum = 0.f;
             // Four taps per round, all reads of a round issued before its first addition.  A
             // tap outside the image (or past the kernel row) reads the slot that holds zero
@@ -408,7 +417,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
                     for (int u = 0; u < 4; u++) sum = __fadd_rn(sum, term[u]);
                 }
             if (lane < 32) {
-                k_lds[ps * 32 + lane] = sum;
+                k_lds[(pg * PS + ps) * 32 + lane] = sum;
                 if (chunk == 0 && live[ps]) k_out[pix[ps]] = sum;
             }
         }
@@ -431,7 +440,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     if constexpr (!PERSIST) alpha_lds[tid] = alpha_early;
 
     // ---- this wave: 64 filters x 32*PS pixels --------------------------------------------------
-    const int oc_sub0 = chunk * (NT / 32) + wave * 2; // first 32-filter block
+    const int oc_sub0 = chunk * (NT / 32) + fw * 2; // first 32-filter block
     const bool wave_has_filters = oc_sub0 * 32 < g.oc; // wave-uniform
 
     v16f acc[2][PS];
@@ -616,7 +625,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     if (!RAW) { // two branches: one select of an LDS and a global pointer would be a flat load
         if (fuse_k) {
 #pragma unroll
-            for (int ps = 0; ps < PS; ps++) kv[ps] = k_lds[ps * 32 + (lane & 31)];
+            for (int ps = 0; ps < PS; ps++) kv[ps] = k_lds[(pg * PS + ps) * 32 + (lane & 31)];
         } else {
 #pragma unroll
             for (int ps = 0; ps < PS; ps++) kv[ps] = kplane[live[ps] ? pix[ps] : 0];
@@ -710,7 +719,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
     uint32_t off2[PS / 2 > 0 ? PS / 2 : 1]; // joined pair q: pixels 64q + lane of one filter
 #pragma unroll
     for (int q = 0; q < PS / 2; q++) {
-        const uint32_t p64 = p_first + q * 64 + lane;
+        const uint32_t p64 = p_wave + q * 64 + lane;
         const uint32_t pc = p64 < p_limit ? p64 : p_limit - 1;
         const uint32_t im = g.div_ohw.div(pc);
         off2[q] = p64 < p_limit
@@ -727,12 +736,12 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
 #pragma unroll
             for (int i4 = 0; i4 < 4; i4++) {
                 // alphas of the four filters 8*i4 + 4*lane_hi + 0..3 of this 32-filter block
-                const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
+                const int ocl4 = (fw * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
                 const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
 #pragma unroll
                 for (int ii = 0; ii < 4; ii++) {
                     const int i = 4 * i4 + ii;
-                    const int f = chunk * NT + (wave * 2 + os) * 32 + 8 * i4 + ii; // lanes 0..31
+                    const int f = chunk * NT + (fw * 2 + os) * 32 + 8 * i4 + ii; // lanes 0..31
                     const uint32_t soff = (uint32_t)f * fstep; // uniform
                     uint32_t v[PS]; // bit patterns of the results in the accumulator layout
 #pragma unroll
@@ -775,17 +784,17 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
         constexpr int STORE_AUX = decltype(policy)::value;
         float *mine = turn_lds + wave * (32 * TURN_ROW);
         const int piece = lane & 7, prow = lane >> 3;
-        const uint32_t left = p_limit - p_first; // pixels of the tile that exist
+        const uint32_t left = p_limit > p_wave ? p_limit - p_wave : 0u; // of this wave's pixels
 #pragma unroll
         for (int os = 0; os < 2; os++) {
-            const uint32_t fpiece = (uint32_t)(chunk * NT + (wave * 2 + os) * 32 + 4 * piece);
+            const uint32_t fpiece = (uint32_t)(chunk * NT + (fw * 2 + os) * 32 + 4 * piece);
             const uint32_t base = fpiece < (uint32_t)g.oc
-                ? ((p_first + (uint32_t)prow) * (uint32_t)g.oc + fpiece) * 4u : DROP;
+                ? ((p_wave + (uint32_t)prow) * (uint32_t)g.oc + fpiece) * 4u : DROP;
 #pragma unroll
             for (int ps = 0; ps < PS; ps++) {
 #pragma unroll
                 for (int i4 = 0; i4 < 4; i4++) {
-                    const int ocl4 = (wave * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
+                    const int ocl4 = (fw * 2 + os) * 32 + 8 * i4 + lane_hi * 4;
                     const v4f al = *reinterpret_cast<const v4f *>(alpha_lds + ocl4);
                     v4i q;
 #pragma unroll
@@ -807,7 +816,7 @@ void conv_tile(const uint32_t *__restrict__ xbits, const v4i *__restrict__ wfrag
             }
         }
     };
-    const bool all_filters = chunk * NT + (wave + 1) * 64 <= g.oc; // wave-uniform
+    const bool all_filters = chunk * NT + (fw + 1) * 64 <= g.oc; // wave-uniform
     if constexpr (!RAW) {
         if (vec4_ok) {
             if (g.stream_dst) store_lines_nhwc(std::integral_constant<int, STORE_STREAMING>{});
@@ -861,8 +870,8 @@ void conv_mfma_fp4_kernel(const uint32_t *__restrict__ xbits, const v4i *__restr
         const uint32_t tile = oc_chunks == 1 ? unit : unit / oc_chunks;
         const int chunk = unit - tile * oc_chunks;
         conv_tile<KS, PS, RAW, PAIR, DEEP>(xbits, wfrag, alpha, kplane, dst, popc, g, max_rows,
-                div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes, tile * (32u * PS),
-                g.npix_out, chunk);
+                div_xw, a_plane, k_out, inv_khw, ic_parts, wfrag_bytes,
+                tile * (32u * PS * (uint32_t)g.mfma_groups), g.npix_out, chunk);
     } else {
         const uint32_t first = xcd * blocks_per_xcd; // pixel blocks of this XCD: [first, last)
         const uint32_t p_limit = min((first + blocks_per_xcd) * 32u, g.npix_out);
@@ -1126,19 +1135,38 @@ int max_tile_rows(const Geometry &g, uint32_t mt, uint32_t step = 0) {
     return most;
 }
 
+// Pixel groups per tile: with 128 filters or fewer only two of a workgroup's four waves would
+// have filters, with 64 or fewer only one; the others then take the same filters on further
+// pixel blocks (see conv_tile).  Not with channel parts.  XNOR_NN_HIP_MFMA_GROUPS=1|2|4
+// overrides (for measurements; more groups than idle waves are not taken).
+int pixel_groups(const Geometry &g) {
+    if (channel_parts(g) > 1) return 1;
+    // two tile sizes in one launch or persistent workgroups asked for by name: one group
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_MIX"))
+        if (e[0] != '0') return 1;
+    if (getenv("XNOR_NN_HIP_MFMA_PERSIST")) return 1;
+    int groups = g.oc <= 64 ? 4 : g.oc <= 128 ? 2 : 1;
+    if (const char *e = getenv("XNOR_NN_HIP_MFMA_GROUPS")) {
+        const int v = atoi(e);
+        if ((v == 1 || v == 2 || v == 4) && v <= groups) groups = v;
+    }
+    return groups;
+}
+
 size_t lds_bytes_for(const Geometry &g, size_t rows, int ps, bool persist = false) {
     const size_t row_bytes = pair_taps(g) ? g.xw * 16
         : channel_parts(g) * steps_per_tap(g) * 32 + ROW_PAD;
     // persistent workgroups: two staging areas for packed words and for mean|x| (conv_tile)
     const size_t stage = persist ? (2 * rows * g.xw * 4 + 2 * (rows + 1) * 4 + 15) & ~(size_t)15 : 0;
+    const int groups = persist ? 1 : g.mfma_groups;
     size_t bytes = TABLE_BYTES + ALPHA_BYTES + stage + (1 + rows) * row_bytes
-        + (rows + 1 + 32 * ps) * sizeof(float);
+        + (rows + 1 + 32 * ps * groups) * sizeof(float);
     if (g.dst_fmt == xnor_nn_data_format_nhwc && (g.oc & 3) == 0) // turn-around rows, 4 waves
         bytes = ((bytes + 15) & ~(size_t)15) + 4 * 32 * TURN_ROW * sizeof(float);
     return bytes;
 }
 size_t lds_bytes(const Geometry &g, int ps) {
-    return lds_bytes_for(g, (size_t)max_tile_rows(g, 32 * ps), ps);
+    return lds_bytes_for(g, (size_t)max_tile_rows(g, 32 * ps * g.mfma_groups), ps);
 }
 
 // 32-pixel blocks per tile, by a model of the kernel's time in core cycles that was fitted to
@@ -1206,13 +1234,14 @@ int pick_ps(const Geometry &g) {
     for (int ps = 4; ps >= 1; ps--) {
         if (lds_bytes(g, ps) > (size_t)LDS_LIMIT) continue;
         if (!tile_fits_registers(g, ps)) continue;
-        const double tiles = (double)((g.npix_out + 32 * ps - 1) / (32 * ps));
+        const uint32_t mt = 32u * ps * g.mfma_groups; // pixels per tile
+        const double tiles = (double)((g.npix_out + mt - 1) / mt);
         // workgroups per compute unit = waves per SIMD; a workgroup whose filters fill fewer
         // than four waves (OC below 256) still takes its slot with all four
         const double per_simd = tiles * chunks * 4 / simds;
         const double busiest = per_simd <= 1 ? 1.0
             : per_simd <= 4 ? (double)(long)(per_simd + 0.999999) : per_simd + 0.5;
-        const double words = (double)max_tile_rows(g, 32 * ps) * g.xw;
+        const double words = (double)max_tile_rows(g, mt) * g.xw;
         const double stream_bound = ps < 2 && per_simd > 1 ? 2.0 : (double)ps;
         const double wave = 3700.0 + 264.0 * words / 256.0 + 1700.0 * ps
             + (ps == 2 ? 70.4 : 64.0) * steps_total * stream_bound;
@@ -1233,7 +1262,8 @@ hipError_t launch_mfma(const Geometry &g, const uint32_t *xbits, const uint32_t 
         const float *alpha, const float *k, float *dst, int32_t *popc,
         const float *a_or_null, float *k_out, hipStream_t s, const KernelEvents &ev) {
     const int chunks = (g.oc + NT - 1) / NT;
-    const uint32_t tiles = (g.npix_out + 32 * PS - 1) / (32 * PS);
+    const uint32_t mt = 32u * PS * (PSB > 0 ? 1u : (uint32_t)g.mfma_groups);
+    const uint32_t tiles = (g.npix_out + mt - 1) / mt;
     const uint32_t units = tiles * chunks;
     uint32_t per_xcd = (units + 7) / 8; // workgroups per XCD
     uint32_t big = 0, blocks = 0;
@@ -1374,6 +1404,9 @@ size_t mfma_weight_bytes(const Geometry &g) {
 }
 
 void mfma_plan(Geometry &g) {
+    // as many pixel groups as idle waves, fewer if even a one-block tile would not fit the LDS
+    for (g.mfma_groups = pixel_groups(g); g.mfma_groups > 1; g.mfma_groups /= 2)
+        if (lds_bytes(g, 1) <= (size_t)LDS_LIMIT) break;
     g.mfma_ps = mfma_tile_blocks(g);
     g.use_mfma = g.mfma_ps > 0 ? 1 : 0;
     g.mfma_steps = g.mfma_pair = g.mfma_rows = 0;
@@ -1401,7 +1434,7 @@ void mfma_plan(Geometry &g) {
     g.mfma_steps = steps_per_tap(g);
     g.mfma_pair = pair_taps(g) ? 1 : 0;
     g.mfma_parts = channel_parts(g);
-    g.mfma_rows = max_tile_rows(g, 32 * g.mfma_ps);
+    g.mfma_rows = max_tile_rows(g, 32 * g.mfma_ps * g.mfma_groups);
     g.mfma_lds = (uint32_t)lds_bytes(g, g.mfma_ps);
     g.mfma_wbytes = (uint32_t)mfma_weight_bytes(g);
     // Few tiles: the small-problem kernel takes the scaled output (the raw accumulators still
@@ -1436,7 +1469,7 @@ void mfma_plan(Geometry &g) {
         fill = e[0] == '3';
     }
     if (getenv("XNOR_NN_HIP_MFMA_PS") || g.mfma_parts > 1 || g.mfma_steps >= 16
-            || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4))
+            || (g.mfma_pair && g.xw >= 5) || !tile_fits_registers(g, 4) || g.mfma_groups > 1)
         mix = fill = false;
     // Persistent workgroups (see the kernel): only on request, XNOR_NN_HIP_MFMA_PERSIST=N with
     // N workgroups per XCD (64 = two per compute unit).  Measured on MI355X they are slower than
@@ -1472,6 +1505,7 @@ void mfma_plan(Geometry &g) {
                     }
                 }
                 g.mfma_persist = 1;
+                g.mfma_groups = 1; // a persistent workgroup walks tiles of one pixel group
                 g.mfma_tiles_per_round = per_round;
                 g.mfma_rounds = best_a + (best_total - 4 * best_a) / 3;
                 g.mfma_reverse = 0;
@@ -1535,6 +1569,9 @@ const char *mfma_kernel_name(const Geometry &g) {
     else if (g.mfma_ps_small > 0)
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d+%d%s>", g.mfma_steps,
                 g.mfma_ps, g.mfma_ps_small, g.mfma_pair ? ",PAIR" : "");
+    else if (g.mfma_groups > 1)
+        snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s,GROUPS=%d>", g.mfma_steps,
+                g.mfma_ps, g.mfma_pair ? ",PAIR" : "", g.mfma_groups);
     else
         snprintf(name, sizeof name, "conv_mfma_fp4_kernel<KS=%d,PS=%d%s>", g.mfma_steps,
                 g.mfma_ps, g.mfma_pair ? ",PAIR" : "");

@@ -70,6 +70,8 @@ struct Geometry {
     int mfma_ps;                // its tile size in 32-pixel blocks (1..4)
     int mfma_ps_small;          // > 0: a launch with two tile sizes; the later workgroups of an
                                 // XCD take this many blocks (see the kernel)
+    int mfma_groups;            // pixel groups per tile (1, 2, 4): with 128 / 64 filters or fewer
+                                // the waves without filters take further pixel blocks instead
     uint32_t mfma_big_per_xcd;  // ... after this many workgroups with mfma_ps blocks,
     uint32_t mfma_blocks_per_xcd; // out of this many pixel blocks per XCD
     int mfma_persist;           // 1: two workgroups per CU stay and walk over the tiles, taking
