@@ -250,7 +250,11 @@ def test_kernel_variants_planned_for_known_shapes(monkeypatch):
     # 6 pixel blocks x 8 filter blocks: fewer (block, block) pairs than compute units
     assert kernel_names((1,) + conv4) == ("binarize_nchw_kernel", "conv_mfma_fp4_small_kernel<KS=6>")
     assert kernel_names((8,) + conv4)[1] == "conv_mfma_fp4_small_kernel<KS=6>"
+    # up to two pairs per compute unit when a wave would walk 48 steps or more (here 54)
+    assert kernel_names((12,) + conv4)[1] == "conv_mfma_fp4_small_kernel<KS=6>"
     assert kernel_names((16,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=1>"
+    # 36 steps: the large-launch kernel from 1.5 pairs per compute unit
+    assert kernel_names((8, 256, 256, 14, 14, 3, 3, 1, 1, 1, 1))[1] == "conv_mfma_fp4_kernel<KS=4,PS=1>"
     # 5.3 pixel blocks per compute unit: two tile sizes in one launch
     assert kernel_names((256,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4+2>"
     assert kernel_names((1024,) + conv4)[1] == "conv_mfma_fp4_kernel<KS=6,PS=4>"

@@ -240,7 +240,15 @@ bool small_kernel_applies(const Geometry &g, int *rows_out, uint32_t *lds_out) {
     // measured on AlexNet conv4 (8 filter blocks): minibatch 1 / 2 / 4 / 8, i.e. 48 to 344
     // pairs, 6.2 / 6.2 / 6.3 / 7.1 us against 7.4 / 7.5 / 7.6 / 7.9 us for the large-launch
     // kernel; minibatch 16 (680 pairs) 8.4 against 8.1 us, minibatch 32 13.5 against 8.7 us
-    bool take = (uint64_t)blocks * subs <= (uint64_t)g.cus + (uint64_t)g.cus / 2;
+    // With long walks (48 steps and more: conv4's 54, 72 for 512 channels) the split of the steps
+    // over four waves still pays at up to two pairs per compute unit: conv4 minibatch 12 (512
+    // pairs) 7.2 against 7.6 us, 512 -> 512 channels on 28x28 minibatch 1 (400 pairs) 8.0 against
+    // 8.6, on 14x14 minibatch 4 7.6 against 8.4, on 7x7 minibatch 20 (496 pairs) 7.5 against
+    // 8.5; with 36 steps (256 channels) the large-launch kernel is ahead there (6.9 against 7.2).
+    const uint64_t pairs = (uint64_t)blocks * subs;
+    const int walk = g.kh * g.kw * g.mfma_steps;
+    bool take = pairs <= (uint64_t)g.cus + (uint64_t)g.cus / 2
+        || (walk >= 48 && pairs <= 2 * (uint64_t)g.cus);
     // a tile size, tile mix or persistent workgroups asked for by name mean the other kernel
     if (getenv("XNOR_NN_HIP_MFMA_PS") || getenv("XNOR_NN_HIP_MFMA_MIX")
             || getenv("XNOR_NN_HIP_MFMA_PERSIST"))
