@@ -144,6 +144,9 @@ def main():
     ap.add_argument("--workload", default="alexnet_conv4_mb256")
     ap.add_argument("--mb", type=int, default=None,
                     help="override the batch size of the workload (experiments only)")
+    ap.add_argument("--shape", default=None, metavar="MB,IC,OC,IH,IW,KH,KW,SH,SW,PH,PW",
+                    help="another layer instead of a named workload (experiments only): N(0,1) "
+                         "input and N(0,0.05) weights of this shape, NCHW/OIHW/NCHW")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-cold", action="store_true",
                     help="skip the leg that rotates through more buffers than the cache holds")
@@ -179,7 +182,18 @@ def main():
         sys.exit("cannot query the HIP device")
     cus, clk_hz = c_cus.value, c_khz.value * 1e3
 
-    d, x, w = synth.make_workload(args.workload, args.mb)
+    if args.shape:
+        dims = [int(v) for v in args.shape.split(",")]
+        if len(dims) != 11 or min(dims) < 0:
+            sys.exit("--shape takes MB,IC,OC,IH,IW,KH,KW,SH,SW,PH,PW")
+        d = dict(zip(("mb", "ic", "oc", "ih", "iw", "kh", "kw", "sh", "sw", "ph", "pw"), dims))
+        x = synth.normal(synth.SEED_SRC, d["mb"] * d["ic"] * d["ih"] * d["iw"]).reshape(
+            d["mb"], d["ic"], d["ih"], d["iw"])
+        w = synth.normal(synth.SEED_WEIGHTS, d["oc"] * d["ic"] * d["kh"] * d["kw"], 0.05).reshape(
+            d["oc"], d["ic"], d["kh"], d["kw"])
+        args.workload = "shape:" + args.shape
+    else:
+        d, x, w = synth.make_workload(args.workload, args.mb)
     wf = work_figures(d)
     xt = torch.from_numpy(x).to(dev)
     wt = torch.from_numpy(w).to(dev)
@@ -361,7 +375,7 @@ def main():
     valu_peak_tops = cus * 64 * clk_hz * 32 / 1e12
     conv_peak = MFMA_FP4_PEAK_TOPS if on_mfma else valu_peak_tops
     conv_tops = wf["exact_ops"] / conv_s / 1e12
-    profiled = args.workload if args.mb is None else "none"
+    profiled = args.workload if args.mb is None and not args.shape else "none"
     # The streaming stage is priced against HBM with its duration inside the cold steps, where
     # its input really comes from HBM; inside the warm steps the input of the default
     # workload is served by the Infinity Cache, which is reported beside it.
